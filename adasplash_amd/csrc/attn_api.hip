@@ -1,0 +1,137 @@
+// C ABI of the attention forward: argument checks, V re-layout launch, kernel dispatch.
+#include "common.h"
+#include "attn_params.h"
+#include <math.h>
+#include "../../include/adasplash_hip.h"
+
+namespace adsp {
+int launch_attn_bf16(const AttnParams& p, int D, int am, hipStream_t s);
+int launch_attn_f16(const AttnParams& p, int D, int am, hipStream_t s);
+int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s);
+
+// Key-major, MFMA-ordered copy of V for the 16-bit path:
+//   vt[bh, d, pos(n)] = v[bh, n, d],  pos(16s + 8a + 4h + r) = 16s + 8h + 4a + r,  zero for n >= N.
+// With this order a lane of the PV product reads its 8 keys {16s + 4h + r, 16s + 8 + 4h + r} of one
+// d row as one 16-byte LDS access.
+__global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
+                                                        int N, int Npad, int D) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint16_t* tile = reinterpret_cast<uint16_t*>(smem);  // [64][D + 2]
+  const int pitch = D + 2;
+  const int kt = blockIdx.x;
+  const size_t bh = blockIdx.y;
+  const uint16_t* vsrc = v + bh * (size_t)N * D;
+  for (int i = threadIdx.x; i < 64 * D; i += 256) {
+    int key = i / D, d = i % D;
+    int gk = kt * 64 + key;
+    tile[key * pitch + d] = gk < N ? vsrc[(size_t)gk * D + d] : (uint16_t)0;
+  }
+  __syncthreads();
+  uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64;
+  for (int i = threadIdx.x; i < 64 * D; i += 256) {
+    int d = i / 64, pos = i % 64;
+    int key = (pos & ~15) | (((pos >> 2) & 1) << 3) | (((pos >> 3) & 1) << 2) | (pos & 3);
+    vdst[(size_t)d * Npad + pos] = tile[key * pitch + d];
+  }
+}
+
+
+static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
+static int mblocks_of(int N) { return (N + kBM - 1) / kBM; }
+static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
+
+static int attn_common(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                       const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
+                       double alpha, int is_causal, int niter, int use_hist, void* workspace, size_t workspace_bytes,
+                       unsigned long long* tile_counts, hipStream_t s) {
+  if (!q || !k || !v || !out) return ADSP_ERR_NULL;
+  if (dtype != ADSP_F32 && dtype != ADSP_BF16 && dtype != ADSP_F16) return ADSP_ERR_DTYPE;
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || Hq % Hkv != 0) return ADSP_ERR_SHAPE;
+  if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return ADSP_ERR_SHAPE;
+  if (mask_words_of(N) > kMaskWords) return ADSP_ERR_SHAPE;
+  if (!(alpha > 1.0) || niter < 0) return ADSP_ERR_UNSUPPORTED;
+  if (varlen && varlen_bits != 32 && varlen_bits != 64) return ADSP_ERR_UNSUPPORTED;
+  if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) return ADSP_ERR_ALIGN;
+
+  AttnParams p;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.vt = nullptr;
+  p.out = out;
+  p.taus = taus;
+  p.bmask = bmask;
+  p.varlen = varlen;
+  p.varlen_bits = varlen_bits;
+  p.tile_counts = tile_counts;
+  p.B = B;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.N = N;
+  p.Npad = npad_of(N);
+  p.n_mblk = mblocks_of(N);
+  p.mask_words = mask_words_of(N);
+  p.niter = niter;
+  p.causal = is_causal ? 1 : 0;
+  p.use_hist = use_hist;
+  p.alpha = (float)alpha;
+  p.c0 = (float)(1.0 / (alpha - 1.0));
+  p.qscale = (float)((alpha - 1.0) / sqrt((double)D));
+  const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
+
+  (void)hipGetLastError();
+  if (dtype != ADSP_F32) {
+    const size_t need = adsp_attn_workspace_bytes(B, Hkv, N, D, dtype);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
+    p.vt = workspace;
+    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hkv)), dim3(256),
+                       (size_t)64 * (D + 2) * 2, s, (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D);
+  }
+  int rc = dtype == ADSP_BF16 ? launch_attn_bf16(p, D, am, s)
+                              : (dtype == ADSP_F16 ? launch_attn_f16(p, D, am, s) : launch_attn_f32(p, D, am, s));
+  if (rc != 0) return ADSP_ERR_LAUNCH;
+  return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
+}
+}  // namespace adsp
+
+extern "C" size_t adsp_attn_workspace_bytes(int B, int Hkv, int N, int D, int dtype) {
+  if (dtype == ADSP_F32 || B <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
+  return (size_t)B * Hkv * D * adsp::npad_of(N) * 2;
+}
+
+extern "C" size_t adsp_attn_bmask_words(int N) {
+  if (N <= 0) return 0;
+  return (size_t)adsp::mblocks_of(N) * adsp::mask_words_of(N);
+}
+
+extern "C" int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                                const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
+                                int niter, void* workspace, size_t workspace_bytes, void* stream) {
+  return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, Hq, Hkv, N, D, dtype, 1.5, 1, niter, 1,
+                           workspace, workspace_bytes, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                                const void* varlen, int varlen_bits, int B, int H, int N, int D, int dtype, double alpha,
+                                int is_causal, int niter, void* workspace, size_t workspace_bytes,
+                                unsigned long long* tile_counts, void* stream) {
+  if (alpha > 2.0) return ADSP_ERR_UNSUPPORTED;
+  return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, H, H, N, D, dtype, alpha, is_causal, niter,
+                           0, workspace, workspace_bytes, tile_counts, (hipStream_t)stream);
+}
+
+extern "C" int adsp_version(void) { return 1; }
+
+extern "C" const char* adsp_status_string(int status) {
+  switch (status) {
+    case ADSP_OK: return "ok";
+    case ADSP_ERR_NULL: return "a required pointer is NULL";
+    case ADSP_ERR_SHAPE: return "a dimension is out of the supported range";
+    case ADSP_ERR_DTYPE: return "unknown element type";
+    case ADSP_ERR_ALIGN: return "a tensor base pointer is not 16-byte aligned";
+    case ADSP_ERR_UNSUPPORTED: return "unsupported parameter combination";
+    case ADSP_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case ADSP_ERR_LAUNCH: return "HIP launch failed";
+  }
+  return "unknown status";
+}

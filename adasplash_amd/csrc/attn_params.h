@@ -1,0 +1,37 @@
+// Launch parameters and tile constants shared by the attention kernel and its C-ABI front end.
+#pragma once
+#include <stdint.h>
+
+namespace adsp {
+
+constexpr int kBM = 128;         // query rows per workgroup
+constexpr int kBN = 64;          // keys per tile
+constexpr int kAttnBins = 8;     // histogram bins of the attention solver
+constexpr int kMaskWords = 512;  // tile-mask capacity per row block: 512 * 32 tiles * 64 keys = 1M keys
+constexpr int kThreads = 256;
+
+enum AttnAlphaMode { ATT_15 = 0, ATT_2 = 1, ATT_GEN = 2 };
+
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;   // fp32 path: row-major V; 16-bit path: unused
+  const void* vt;  // 16-bit path: key-major permuted copy of V, [B*Hkv, D, Npad]
+  void* out;
+  float* taus;
+  int32_t* bmask;
+  const void* varlen;
+  int varlen_bits;
+  unsigned long long* tile_counts;
+  int B, Hq, Hkv, N, Npad;
+  int n_mblk;      // row blocks per (b, h)
+  int mask_words;  // int32 words per row block in bmask
+  int niter;
+  int causal;
+  int use_hist;
+  float qscale;  // (alpha - 1) / sqrt(D)
+  float alpha;
+  float c0;  // 1 / (alpha - 1)
+};
+
+}  // namespace adsp

@@ -1,0 +1,71 @@
+// Shared device helpers for the gfx950 kernels: element types, wave64 reductions, conversions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace adsp {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // a 16-byte global/LDS access
+
+struct bf16_t { uint16_t bits; };  // storage-only tags; arithmetic is always fp32
+struct f16_t { uint16_t bits; };
+
+template <typename T> struct elem_traits;
+template <> struct elem_traits<float> { static constexpr int kBytes = 4; static constexpr int kVec = 4; };
+template <> struct elem_traits<bf16_t> { static constexpr int kBytes = 2; static constexpr int kVec = 8; };
+template <> struct elem_traits<f16_t> { static constexpr int kBytes = 2; static constexpr int kVec = 8; };
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);  // v_cvt_pk_bf16_f32, round to nearest even
+}
+__device__ __forceinline__ float f16_bits_to_float(uint32_t b) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+__device__ __forceinline__ uint32_t float_to_f16_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// Two fp32 -> one dword of packed 16-bit elements (low half = a).
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+}
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t w) { return f16_bits_to_float(w & 0xffffu); }
+template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t w) { return f16_bits_to_float(w >> 16); }
+
+// ---- wave64 butterflies ---------------------------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+}  // namespace adsp

@@ -1,0 +1,393 @@
+// Row-wise alpha-entmax forward / backward for gfx950.
+//
+// Forward: y[r, j] = [(alpha-1) x[r, j] - tau_r]_+^(1/(alpha-1)).  The kernel is HBM-bound: a row is read
+// from HBM exactly once (16-byte loads, the whole row then lives in registers), every solver pass
+// (max, histogram bracket, refinement) runs on the register copy with wave64 butterflies (plus one LDS
+// exchange when a row spans four waves), and the result is written once.  Rows that do not fit in
+// registers, or whose base is not 16-byte aligned, take a streaming variant that re-reads the row
+// (from L2) per pass.  Semantics follow adasplash/triton_entmax_v2.py:363-536.
+#include "common.h"
+#include "solver.h"
+#include "../../include/adasplash_hip.h"
+
+namespace adsp {
+
+constexpr int kRowBins = 4;  // histogram bins of the standalone rows kernel (triton_entmax_v2.py:386)
+
+enum AlphaMode { AM_15 = 0, AM_2 = 1, AM_GEN = 2 };
+
+struct RowsParams {
+  const void* x;
+  void* y;
+  long long rows, cols;
+  float scale;  // alpha - 1
+  float c0;     // 1 / (alpha - 1)
+  int n_iter;
+  int use_hist;
+  int allow_halley, allow_newton;
+};
+
+// ---- reductions across the TPR threads that share a row ---------------------------------------------
+template <int TPR> __device__ __forceinline__ float row_max(float v, float* sm) {
+  v = wave_max(v);
+  if constexpr (TPR > 64) {
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = sm[0];
+#pragma unroll
+    for (int w = 1; w < TPR / 64; ++w) v = fmaxf(v, sm[w]);
+  }
+  return v;
+}
+template <int TPR, int K> __device__ __forceinline__ void row_sum(float (&v)[K], float* sm) {
+#pragma unroll
+  for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
+  if constexpr (TPR > 64) {
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) sm[(threadIdx.x >> 6) * K + k] = v[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      float s = sm[k];
+#pragma unroll
+      for (int w = 1; w < TPR / 64; ++w) s += sm[w * K + k];
+      v[k] = s;
+    }
+  }
+}
+
+template <int AM> __device__ __forceinline__ float prob(float u, float c0) {
+  // u = z - tau (may be <= 0)
+  if constexpr (AM == AM_2) return fmaxf(u, 0.f);
+  if constexpr (AM == AM_15) {
+    float r = fmaxf(u, 0.f);
+    return r * r;
+  }
+  return u > 0.f ? fast_exp2(fast_log2(u) * c0) : 0.f;
+}
+
+template <int AM> __device__ __forceinline__ void accum_stats(float u, float c0, float (&a)[3]) {
+  if constexpr (AM == AM_2) {
+    a[0] += fmaxf(u, 0.f);
+    a[1] += u > 0.f ? 1.f : 0.f;
+  } else if constexpr (AM == AM_15) {
+    float r = fmaxf(u, 0.f);
+    a[0] = fmaf(r, r, a[0]);
+    a[1] += r;
+    a[2] += u > 0.f ? 1.f : 0.f;
+  } else {
+    if (u > 0.f) {
+      float uc = fmaxf(u, 1e-6f);  // same clamp as the reference's masked power (triton_entmax_v2.py:35-39)
+      float lg = fast_log2(uc);
+      a[0] += fast_exp2(lg * c0);
+      a[1] += fast_exp2(lg * (c0 - 1.f));
+      a[2] += fast_exp2(lg * (c0 - 2.f));
+    }
+  }
+}
+
+// The whole per-row solve, generic over how the row's scaled elements z are visited.
+// `Row::for_each(f)` calls f(z) for every element this thread owns (invalid slots yield -inf).
+template <int AM, int TPR, typename Row>
+__device__ __forceinline__ float solve_row(const Row& row, const RowsParams& p, float* sm) {
+  float m = -INFINITY;
+  row.for_each([&](float z) { m = fmaxf(m, z); });
+  m = row_max<TPR>(m, sm);
+
+  Bracket br;
+  if (AM != AM_GEN && p.use_hist) {
+    const float t_shift = m - 1.f;
+    float cnt[kRowBins];
+#pragma unroll
+    for (int b = 0; b < kRowBins; ++b) cnt[b] = 0.f;
+    row.for_each([&](float z) {
+      float pr = (z - t_shift) * (float)kRowBins;
+      if (pr >= 0.f) {
+#pragma unroll
+        for (int b = 0; b < kRowBins; ++b) {
+          bool in = (b == kRowBins - 1) ? (pr >= (float)b) : (pr >= (float)b && pr < (float)(b + 1));
+          cnt[b] += in ? 1.f : 0.f;
+        }
+      }
+    });
+    row_sum<TPR, kRowBins>(cnt, sm);
+    br.lo = (AM == AM_15) ? hist_bracket_alpha15<kRowBins>(cnt, t_shift) : hist_bracket_alpha2<kRowBins>(cnt, t_shift);
+    br.lo = fmaxf(br.lo, t_shift);
+    br.hi = fminf(br.lo + 1.f / (float)kRowBins, m);
+    br.t = hist_start_point<kRowBins>(cnt, t_shift, br.lo, br.hi);
+  } else {
+    br.lo = m - 1.f;
+    br.hi = m;
+    br.t = 0.5f * (br.lo + br.hi);
+  }
+
+  // n_iter refinement steps as requested, then keep stepping (the row is in registers, so a step costs
+  // no memory traffic) until |f| is at rounding level or the extra-step cap is reached.
+  float t_prev = br.t, f_prev = 0.f;
+  const int kExtra = 12;
+  for (int it = 0; it < p.n_iter + kExtra; ++it) {
+    float a[3] = {0.f, 0.f, 0.f};
+    const float t = br.t;
+    row.for_each([&](float z) { accum_stats<AM>(z - t, p.c0, a); });
+    row_sum<TPR, 3>(a, sm);
+    if (it >= p.n_iter && fabsf(a[0] - 1.f) <= 2e-6f) break;
+    hybrid_step(br, a[0], a[1], a[2], p.c0, p.allow_halley, p.allow_newton, it > 0, t_prev, f_prev);
+  }
+  return br.t;
+}
+
+// ---- register-resident rows ------------------------------------------------------------------------
+template <typename T, int NCHUNK, int TPR> struct RegRow {
+  static constexpr int kVec = elem_traits<T>::kVec;
+  float z[NCHUNK * kVec];
+  template <typename F> __device__ __forceinline__ void for_each(F f) const {
+#pragma unroll
+    for (int i = 0; i < NCHUNK * kVec; ++i) f(z[i]);
+  }
+};
+
+template <typename T, int AM, int NCHUNK, int TPR>
+__global__ __launch_bounds__(256) void entmax_rows_reg_kernel(RowsParams p) {
+  constexpr int kVec = elem_traits<T>::kVec;
+  constexpr int kRowsPerBlock = 256 / TPR;
+  __shared__ float sm[32];
+  const int tid = threadIdx.x;
+  const int t_in_row = tid % TPR;
+  long long row = (long long)blockIdx.x * kRowsPerBlock + tid / TPR;
+  // TPR == 256: one row per block, every thread is active.  TPR == 64: a wave owns a row, and a wave
+  // past the last row simply leaves (no block-level barrier is used in that configuration).
+  if (row >= p.rows) return;
+
+  const long long nvec = p.cols / kVec;
+  const u32x4* xrow = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.x) +
+                                                     (size_t)row * p.cols * elem_traits<T>::kBytes);
+  u32x4* yrow = reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.y) + (size_t)row * p.cols * elem_traits<T>::kBytes);
+
+  RegRow<T, NCHUNK, TPR> r;
+  u32x4 raw[NCHUNK];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    long long vi = (long long)c * TPR + t_in_row;
+    if (vi < nvec) raw[c] = __builtin_nontemporal_load(xrow + vi);
+  }
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    long long vi = (long long)c * TPR + t_in_row;
+    const bool ok = vi < nvec;
+    const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+    if constexpr (kVec == 4) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r.z[c * 4 + e] = ok ? __builtin_bit_cast(float, w[e]) * p.scale : -INFINITY;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        r.z[c * 8 + 2 * e] = ok ? unpack_lo<T>(w[e]) * p.scale : -INFINITY;
+        r.z[c * 8 + 2 * e + 1] = ok ? unpack_hi<T>(w[e]) * p.scale : -INFINITY;
+      }
+    }
+  }
+
+  const float tau = solve_row<AM, TPR>(r, p, sm);
+
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    long long vi = (long long)c * TPR + t_in_row;
+    if (vi < nvec) {
+      u32x4 o;
+      if constexpr (kVec == 4) {
+        o.x = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 0] - tau, p.c0));
+        o.y = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 1] - tau, p.c0));
+        o.z = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 2] - tau, p.c0));
+        o.w = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 3] - tau, p.c0));
+      } else {
+        o.x = pack2<T>(prob<AM>(r.z[c * 8 + 0] - tau, p.c0), prob<AM>(r.z[c * 8 + 1] - tau, p.c0));
+        o.y = pack2<T>(prob<AM>(r.z[c * 8 + 2] - tau, p.c0), prob<AM>(r.z[c * 8 + 3] - tau, p.c0));
+        o.z = pack2<T>(prob<AM>(r.z[c * 8 + 4] - tau, p.c0), prob<AM>(r.z[c * 8 + 5] - tau, p.c0));
+        o.w = pack2<T>(prob<AM>(r.z[c * 8 + 6] - tau, p.c0), prob<AM>(r.z[c * 8 + 7] - tau, p.c0));
+      }
+      __builtin_nontemporal_store(o, yrow + vi);
+    }
+  }
+}
+
+// ---- streaming rows (any length / alignment): one 256-thread block per row, scalar accesses --------
+template <typename T> __device__ __forceinline__ float load_elem(const void* base, size_t i);
+template <> __device__ __forceinline__ float load_elem<float>(const void* b, size_t i) { return ((const float*)b)[i]; }
+template <> __device__ __forceinline__ float load_elem<bf16_t>(const void* b, size_t i) {
+  return bf16_bits_to_float(((const uint16_t*)b)[i]);
+}
+template <> __device__ __forceinline__ float load_elem<f16_t>(const void* b, size_t i) {
+  return f16_bits_to_float(((const uint16_t*)b)[i]);
+}
+template <typename T> __device__ __forceinline__ void store_elem(void* base, size_t i, float v);
+template <> __device__ __forceinline__ void store_elem<float>(void* b, size_t i, float v) { ((float*)b)[i] = v; }
+template <> __device__ __forceinline__ void store_elem<bf16_t>(void* b, size_t i, float v) {
+  ((uint16_t*)b)[i] = (uint16_t)float_to_bf16_bits(v);
+}
+template <> __device__ __forceinline__ void store_elem<f16_t>(void* b, size_t i, float v) {
+  ((uint16_t*)b)[i] = (uint16_t)float_to_f16_bits(v);
+}
+
+template <typename T> struct StreamRow {
+  const void* x;
+  size_t base;
+  long long cols;
+  float scale;
+  template <typename F> __device__ __forceinline__ void for_each(F f) const {
+    for (long long j = threadIdx.x; j < cols; j += 256) f(load_elem<T>(x, base + j) * scale);
+  }
+};
+
+template <typename T, int AM> __global__ __launch_bounds__(256) void entmax_rows_stream_kernel(RowsParams p) {
+  __shared__ float sm[32];
+  for (long long row = blockIdx.x; row < p.rows; row += gridDim.x) {
+    StreamRow<T> r{p.x, (size_t)row * p.cols, p.cols, p.scale};
+    const float tau = solve_row<AM, 256>(r, p, sm);
+    for (long long j = threadIdx.x; j < p.cols; j += 256) {
+      float z = load_elem<T>(p.x, r.base + j) * p.scale;
+      store_elem<T>(p.y, r.base + j, prob<AM>(z - tau, p.c0));
+    }
+  }
+}
+
+// ---- backward: dx = u*dy - (sum u*dy / sum u) * u, u = y^(2-alpha) on y > 0 (triton_entmax_v2.py:541-617)
+template <typename T, int AM> __global__ __launch_bounds__(256) void entmax_rows_bwd_kernel(
+    const void* y, const void* dy, void* dx, long long rows, long long cols, float cf) {
+  __shared__ float sm[32];
+  for (long long row = blockIdx.x; row < rows; row += gridDim.x) {
+    const size_t base = (size_t)row * cols;
+    float s[2] = {0.f, 0.f};
+    for (long long j = threadIdx.x; j < cols; j += 256) {
+      float yy = load_elem<T>(y, base + j);
+      float g = load_elem<T>(dy, base + j);
+      float u = 0.f;
+      if (yy > 0.f) u = (AM == AM_2) ? 1.f : (AM == AM_15 ? sqrtf(yy) : fast_exp2(fast_log2(fmaxf(yy, 1e-6f)) * cf));
+      s[0] = fmaf(u, g, s[0]);
+      s[1] += u;
+    }
+    row_sum<256, 2>(s, sm);
+    const float q = s[0] / s[1];
+    for (long long j = threadIdx.x; j < cols; j += 256) {
+      float yy = load_elem<T>(y, base + j);
+      float g = load_elem<T>(dy, base + j);
+      float u = 0.f;
+      if (yy > 0.f) u = (AM == AM_2) ? 1.f : (AM == AM_15 ? sqrtf(yy) : fast_exp2(fast_log2(fmaxf(yy, 1e-6f)) * cf));
+      store_elem<T>(dx, base + j, u * g - q * u);
+    }
+    __syncthreads();
+  }
+}
+
+// ---- host dispatch ---------------------------------------------------------------------------------
+template <typename T, int AM, int NCHUNK, int TPR> static void launch_reg(const RowsParams& p, hipStream_t s) {
+  constexpr int rpb = 256 / TPR;
+  long long blocks = (p.rows + rpb - 1) / rpb;
+  hipLaunchKernelGGL((entmax_rows_reg_kernel<T, AM, NCHUNK, TPR>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+}
+
+template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool aligned, int force_tpr, hipStream_t s) {
+  constexpr int kVec = elem_traits<T>::kVec;
+  const long long nvec = p.cols / kVec;
+  const bool can_reg = aligned && (p.cols % kVec == 0) && p.rows < (1ll << 31);
+  if (can_reg) {
+    const long long c64 = (nvec + 63) / 64, c256 = (nvec + 255) / 256;
+    // A wave per row while the row fits in <= 64 registers per lane; four waves per row beyond that.
+    int tpr = (c64 * kVec <= 64) ? 64 : 256;
+    if (force_tpr == 64 && c64 <= 32) tpr = 64;
+    if (force_tpr == 256) tpr = 256;
+    if (tpr == 64) {
+      if (c64 <= 1) return launch_reg<T, AM, 1, 64>(p, s);
+      if (c64 <= 2) return launch_reg<T, AM, 2, 64>(p, s);
+      if (c64 <= 4) return launch_reg<T, AM, 4, 64>(p, s);
+      if (c64 <= 8) return launch_reg<T, AM, 8, 64>(p, s);
+      if (c64 <= 16) return launch_reg<T, AM, 16, 64>(p, s);
+      if (c64 <= 32) return launch_reg<T, AM, 32, 64>(p, s);
+    } else {
+      if (c256 <= 1) return launch_reg<T, AM, 1, 256>(p, s);
+      if (c256 <= 2) return launch_reg<T, AM, 2, 256>(p, s);
+      if (c256 <= 4) return launch_reg<T, AM, 4, 256>(p, s);
+      if (c256 <= 8) return launch_reg<T, AM, 8, 256>(p, s);
+      if (c256 <= 16) return launch_reg<T, AM, 16, 256>(p, s);
+      if (c256 <= 32) return launch_reg<T, AM, 32, 256>(p, s);
+    }
+  }
+  long long blocks = p.rows < 65536 ? p.rows : 65536;
+  hipLaunchKernelGGL((entmax_rows_stream_kernel<T, AM>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+}
+
+template <typename T> static void launch_fwd_am(const RowsParams& p, int am, bool aligned, int force_tpr, hipStream_t s) {
+  if (am == AM_15) return launch_fwd<T, AM_15>(p, aligned, force_tpr, s);
+  if (am == AM_2) return launch_fwd<T, AM_2>(p, aligned, force_tpr, s);
+  return launch_fwd<T, AM_GEN>(p, aligned, force_tpr, s);
+}
+
+template <typename T> static void launch_bwd_am(const void* y, const void* dy, void* dx, long long rows, long long cols,
+                                                int am, float cf, hipStream_t s) {
+  long long blocks = rows < 65536 ? rows : 65536;
+  if (am == AM_15)
+    hipLaunchKernelGGL((entmax_rows_bwd_kernel<T, AM_15>), dim3((unsigned)blocks), dim3(256), 0, s, y, dy, dx, rows, cols, cf);
+  else if (am == AM_2)
+    hipLaunchKernelGGL((entmax_rows_bwd_kernel<T, AM_2>), dim3((unsigned)blocks), dim3(256), 0, s, y, dy, dx, rows, cols, cf);
+  else
+    hipLaunchKernelGGL((entmax_rows_bwd_kernel<T, AM_GEN>), dim3((unsigned)blocks), dim3(256), 0, s, y, dy, dx, rows, cols, cf);
+}
+
+static int alpha_mode(double alpha) { return alpha == 1.5 ? AM_15 : (alpha == 2.0 ? AM_2 : AM_GEN); }
+
+}  // namespace adsp
+
+// Tuning knob for experiments (0 = automatic, 64 = a wave per row, 256 = a block per row).
+static int g_rows_force_tpr = 0;
+extern "C" void adsp_debug_set_rows_threads_per_row(int tpr) { g_rows_force_tpr = tpr; }
+
+extern "C" int adsp_entmax_rows_fwd(const void* x, void* y, int64_t rows, int64_t cols, int dtype, double alpha,
+                                    int n_iter, int use_histogram, int fast_math, void* stream) {
+  using namespace adsp;
+  (void)fast_math;
+  if (rows < 0 || cols < 0) return ADSP_ERR_SHAPE;
+  if (rows == 0 || cols == 0) return ADSP_OK;
+  if (!x || !y) return ADSP_ERR_NULL;
+  if (!(alpha > 1.0) || n_iter < 0) return ADSP_ERR_UNSUPPORTED;
+  if (dtype != ADSP_F32 && dtype != ADSP_BF16 && dtype != ADSP_F16) return ADSP_ERR_DTYPE;
+  RowsParams p;
+  p.x = x;
+  p.y = y;
+  p.rows = rows;
+  p.cols = cols;
+  p.scale = (float)(alpha - 1.0);
+  p.c0 = (float)(1.0 / (alpha - 1.0));
+  p.n_iter = n_iter;
+  p.use_hist = use_histogram ? 1 : 0;
+  p.allow_halley = alpha <= 1.5;
+  p.allow_newton = alpha <= 2.0;
+  const int am = alpha_mode(alpha);
+  const bool aligned = (((uintptr_t)x | (uintptr_t)y) & 15) == 0;
+  hipStream_t s = (hipStream_t)stream;
+  (void)hipGetLastError();
+  if (dtype == ADSP_F32) launch_fwd_am<float>(p, am, aligned, g_rows_force_tpr, s);
+  else if (dtype == ADSP_BF16) launch_fwd_am<bf16_t>(p, am, aligned, g_rows_force_tpr, s);
+  else launch_fwd_am<f16_t>(p, am, aligned, g_rows_force_tpr, s);
+  return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
+}
+
+extern "C" int adsp_entmax_rows_bwd(const void* y, const void* dy, void* dx, int64_t rows, int64_t cols, int dtype,
+                                    double alpha, void* stream) {
+  using namespace adsp;
+  if (rows < 0 || cols < 0) return ADSP_ERR_SHAPE;
+  if (rows == 0 || cols == 0) return ADSP_OK;
+  if (!y || !dy || !dx) return ADSP_ERR_NULL;
+  if (!(alpha > 1.0)) return ADSP_ERR_UNSUPPORTED;
+  const int am = alpha_mode(alpha);
+  const float cf = (float)(2.0 - alpha);
+  hipStream_t s = (hipStream_t)stream;
+  (void)hipGetLastError();
+  if (dtype == ADSP_F32) launch_bwd_am<float>(y, dy, dx, rows, cols, am, cf, s);
+  else if (dtype == ADSP_BF16) launch_bwd_am<bf16_t>(y, dy, dx, rows, cols, am, cf, s);
+  else if (dtype == ADSP_F16) launch_bwd_am<f16_t>(y, dy, dx, rows, cols, am, cf, s);
+  else return ADSP_ERR_DTYPE;
+  return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
+}

@@ -1,0 +1,111 @@
+/*
+ * adasplash_hip.h -- C ABI of the MI355X (gfx950) sparse entmax attention library.
+ *
+ * Every entry point takes raw device pointers, sizes and scalars, enqueues its kernels on the
+ * HIP stream it is given (a hipStream_t passed as void*; NULL = the default stream), never
+ * synchronises, never allocates and keeps no state between calls.  The caller owns every buffer,
+ * including the workspace.  The return value is an adsp_status; nothing is thrown across the ABI.
+ *
+ * The entry points replace the Triton launches inside the reference's autograd wrappers (the
+ * reference has no FFI of its own; these are the calls a binding would make in their place):
+ *
+ *   adsp_entmax_rows_fwd  <- _entmax_triton.forward -> _fwd_entmax
+ *                            (adasplash/triton_entmax_v2.py:624-664, kernel :363-536)
+ *   adsp_entmax_rows_bwd  <- _entmax_triton.backward -> _bwd_entmax
+ *                            (adasplash/triton_entmax_v2.py:667-687, kernel :541-617)
+ *   adsp_attn_v2_fwd      <- _sparse_attention.forward -> _get_tau, _get_tau_v2, _get_tau_v3,
+ *                            _get_output (adasplash/adasplash_v2.py:1243-1438)
+ *   adsp_attn_v1_fwd      <- _sparse_attention.forward -> _get_tau,
+ *                            compute_bidxs_and_cubcounts, _get_output
+ *                            (adasplash/adasplash_block_mask.py:941-1076)
+ */
+#ifndef ADASPLASH_HIP_H
+#define ADASPLASH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  ADSP_OK = 0,
+  ADSP_ERR_NULL = 1,        /* a required pointer is NULL */
+  ADSP_ERR_SHAPE = 2,       /* a dimension is out of the supported range */
+  ADSP_ERR_DTYPE = 3,       /* unknown element type */
+  ADSP_ERR_ALIGN = 4,       /* a tensor base pointer is not 16-byte aligned */
+  ADSP_ERR_UNSUPPORTED = 5, /* parameter combination the kernels do not implement */
+  ADSP_ERR_WORKSPACE = 6,   /* workspace missing or smaller than adsp_attn_workspace_bytes() */
+  ADSP_ERR_LAUNCH = 7       /* the HIP runtime refused a launch (hipGetLastError() != success) */
+} adsp_status;
+
+/* Element types of q/k/v/out and x/y. */
+typedef enum { ADSP_F32 = 0, ADSP_BF16 = 1, ADSP_F16 = 2 } adsp_dtype;
+
+/* Library ABI version (bumped when a signature changes). */
+int adsp_version(void);
+
+/* Static, NUL-terminated description of a status code. */
+const char* adsp_status_string(int status);
+
+/*
+ * Row-wise alpha-entmax over the last dimension: y[r, :] = [(alpha-1) x[r, :] - tau_r]_+^(1/(alpha-1)).
+ *   x, y      : contiguous [rows, cols] arrays of `dtype`; y is fully overwritten (zeros included).
+ *   alpha     : > 1.  n_iter : refinement steps after initialisation (>= 0).
+ *   use_histogram : non-zero = histogram initialisation of tau (honoured for alpha in {1.5, 2}).
+ *   fast_math : accepted for signature parity; the generic-alpha power always uses exp2/log2.
+ * Replaces the launch at adasplash/triton_entmax_v2.py:650-658.
+ */
+int adsp_entmax_rows_fwd(const void* x, void* y, int64_t rows, int64_t cols, int dtype, double alpha,
+                         int n_iter, int use_histogram, int fast_math, void* stream);
+
+/*
+ * Backward of the above: dx = u*dy - (sum(u*dy)/sum(u)) * u with u = y^(2-alpha) on the support.
+ * Replaces the launch at adasplash/triton_entmax_v2.py:678-685.
+ */
+int adsp_entmax_rows_bwd(const void* y, const void* dy, void* dx, int64_t rows, int64_t cols, int dtype,
+                         double alpha, void* stream);
+
+/*
+ * Bytes of scratch the attention entry points need for these dimensions (a key-major copy of V for
+ * the 16-bit types; 0 for fp32).  The buffer must be 256-byte aligned device memory.
+ */
+size_t adsp_attn_workspace_bytes(int B, int Hkv, int N, int D, int dtype);
+
+/* Number of int32 words per (batch, head) the block mask needs: n_row_blocks * words_per_row. */
+size_t adsp_attn_bmask_words(int N);
+
+/*
+ * AdaSplash-2 forward: causal entmax-1.5 attention with GQA and right-padded variable lengths.
+ *   q, out : [B, Hq, N, D]; k, v : [B, Hkv, N, D], contiguous, Hq % Hkv == 0, D in {16,32,64,128,256}.
+ *   taus   : [B, Hq, N] fp32, receives the per-row threshold (rows past the valid length untouched).
+ *   bmask  : [B, Hq, adsp_attn_bmask_words(N)] int32, receives the per-(128-row, 64-key) tile mask,
+ *            bit (c % 32) of word c / 32 of a row block = key tile c holds a non-zero probability.
+ *   varlen : NULL, or [B] valid lengths as int32 (varlen_bits = 32) or int64 (varlen_bits = 64);
+ *            keys >= length are masked, output rows >= length are written as zeros.
+ *   niter  : Halley/bisection refinement passes after the histogram bracket (>= 0).
+ * Replaces the four launches at adasplash/adasplash_v2.py:1288-1419.
+ */
+int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                     const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
+                     int niter, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * AdaSplash-1 (block-mask) forward: alpha-entmax attention for any alpha in (1, 2], causal or not,
+ * right-padded variable lengths, no GQA (q, k, v share [B, H, N, D]).
+ *   tile_counts : NULL, or 2 device uint64 that are incremented by {16x16 score tiles inside the
+ *                 causal/valid domain, those that hold a non-zero probability} (for sparsity reports).
+ * Other arguments as in adsp_attn_v2_fwd.  Replaces the launches at
+ * adasplash/adasplash_block_mask.py:978-1003 and :1024-1054 plus the torch-side list building
+ * (:298-320).
+ */
+int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                     const void* varlen, int varlen_bits, int B, int H, int N, int D, int dtype, double alpha,
+                     int is_causal, int niter, void* workspace, size_t workspace_bytes,
+                     unsigned long long* tile_counts, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ADASPLASH_HIP_H */
