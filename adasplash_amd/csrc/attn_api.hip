@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restri
 
 
 static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
-static int mblocks_of(int N) { return (N + kBM - 1) / kBM; }
+static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }
 static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
 
 static int attn_common(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,

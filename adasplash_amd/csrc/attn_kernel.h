@@ -1,23 +1,28 @@
 // Fused sparse entmax attention forward for gfx950 (one kernel: threshold solver + output).
 //
 // Work decomposition
-//   workgroup = 256 threads = 4 waves, owns kBM = 128 consecutive query rows of one (batch, head);
-//   wave w owns rows [32w, 32w+32); inside a wave, lane l holds query row (l & 31) and, of every
-//   32-key block, the 16 keys {8g + 4(l >> 5) + r : g, r in 0..3} -- the C layout of the 32x32 MFMA when
-//   the product is taken as S^T = K Q^T.  All per-row quantities (max, histogram, Halley sums, tau,
-//   sum of p) are therefore lane-local accumulators that need one cross-lane add (lane ^ 32) per pass.
-//   K tiles (64 keys) and V tiles are staged through LDS, double-buffered, shared by the four waves.
+//   workgroup = NW waves (8, or 4 for the register-heavy shapes), owns 32*NW consecutive query rows of
+//   one (batch, head); wave w owns rows [32w, 32w+32); inside a wave, lane l holds query row (l & 31)
+//   and, of every 32-key block, the 16 keys {8g + 4(l >> 5) + r : g, r in 0..3} -- the C layout of the
+//   32x32 MFMA when the product is taken as S^T = K Q^T.  All per-row quantities (max, histogram,
+//   Halley sums, tau, sum of p) are therefore lane-local accumulators that need one cross-lane add
+//   (lane ^ 32) per pass.
+//   K tiles (64 keys) and V tiles go HBM/L2 -> LDS with direct 16-byte loads (no staging registers),
+//   double-buffered: the next tile is in flight while the current one is multiplied.  Rows are
+//   XOR-swizzled in 16-byte chunks instead of padded, so the DMA can write contiguous kilobytes and the
+//   ds_read_b128 of 16 consecutive rows still covers all 64 banks.
 //
-// Passes over the K tiles of a row block (every pass recomputes S^T with MFMA, scores never leave
-// registers):
+// Passes over the K tiles of a row block (every pass recomputes S^T with MFMA; scores never leave
+// registers).  s = q.k is kept in raw units and the (alpha-1)/sqrt(D) scale is applied to per-row
+// scalars only, so the MFMA operands are the caller's q and k bit for bit:
 //   A  row max m                                          -> tau in [m - 1, m - n^(1-alpha)]
 //   B  (alpha = 1.5 / 2) 8-bin histogram of z - (m - 1)   -> bracket [lo, lo + 1/8]; tile mask {z > m-1}
-//   C  x niter: sums of u^c0, u^(c0-1), u^(c0-2)          -> Halley / Newton / bisection step; tile mask
-//                                                           refined to {z > lo}
+//   C  x niter: sums of u^c0, u^(c0-1), u^(c0-2)          -> Halley / Newton / bisection step; the last
+//                                                           one refines the tile mask to {z > lo}
 //   D  p = [z - tau]_+^c0, out += P V over masked tiles, divided by sum p at the end.
 // The accumulator of the S^T MFMA is initialised with -tau (resp. -(m-1)), so z - tau costs no VALU op.
 //
-// The 16-bit path consumes V through a key-major copy (see vt_layout_kernel) so that the PV product
+// The 16-bit path consumes V through a key-major copy (vt_layout_kernel) so that the PV product
 // out^T = V^T P^T can take P^T straight from the S^T accumulators without an LDS round trip.
 #pragma once
 #include "common.h"
@@ -28,6 +33,7 @@ namespace adsp {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 
@@ -42,46 +48,71 @@ template <> __device__ __forceinline__ f32x16 mfma_16bit<f16_t>(u32x4 a, u32x4 b
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
 }
 
-// LDS geometry of one K tile and one V tile.
+// 16-byte global -> LDS copy per lane: lane i of the wave writes LDS bytes [16 i, 16 i + 16) after the
+// wave-uniform base `lds`, from its own global address.
+__device__ __forceinline__ void dma16(const void* gsrc, void* lds) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
+// Tile geometry.  A tile row has kC 16-byte chunks; chunk c of row r is stored at chunk position
+// c ^ sw(r), with sw chosen so that 16 consecutive rows reading the same logical chunk touch 16 different
+// 16-byte bank groups.
+template <int ROW_BYTES> struct Swz {
+  static constexpr int kC = ROW_BYTES / 16;
+  static constexpr int kShift = kC >= 16 ? 0 : (kC == 8 ? 1 : (kC == 4 ? 2 : (kC == 2 ? 3 : 4)));
+  static constexpr int kMask = (kC >= 16 ? 16 : kC) - 1;
+  __device__ static __forceinline__ int sw(int row) { return (row >> kShift) & kMask; }
+  __device__ static __forceinline__ int off(int row, int c) { return row * ROW_BYTES + ((c ^ sw(row)) << 4); }
+};
+
 template <typename T, int D> struct TileGeo {
   static constexpr bool k16 = is16<T>::value;
   static constexpr int kEB = k16 ? 2 : 4;
-  static constexpr int kKPitch = D * kEB + 16;  // bytes per key row (+16 B pad against bank conflicts)
-  static constexpr int kKTile = kBN * kKPitch;
-  static constexpr int kVPitch = k16 ? (kBN * 2 + 16) : (D * 4 + 16);
+  static constexpr int kKRow = D * kEB;                // bytes per key row of the K tile
+  static constexpr int kKTile = kBN * kKRow;
+  static constexpr int kVRow = k16 ? kBN * 2 : D * 4;  // 16-bit: V^T tile [D][64 keys]; fp32: V tile [64][D]
   static constexpr int kVRows = k16 ? D : kBN;
-  static constexpr int kVTile = kVRows * kVPitch;
-  static constexpr int kMaskBytes = 2 * kMaskWords * 4;
-  static constexpr int kNBuf = (2 * (kKTile + kVTile) + kMaskBytes <= 150 * 1024) ? 2 : 1;
-  static constexpr int kLdsBytes = kNBuf * (kKTile + kVTile) + kMaskBytes;
-  static constexpr int kKChunksPerRow = D * kEB / 16;
-  static constexpr int kKChunks = kBN * kKChunksPerRow;
-  static constexpr int kKPerThread = (kKChunks + kThreads - 1) / kThreads;
-  static constexpr int kVChunksPerRow = k16 ? 8 : (D * 4 / 16);
-  static constexpr int kVChunks = kVRows * kVChunksPerRow;
-  static constexpr int kVPerThread = (kVChunks + kThreads - 1) / kThreads;
+  static constexpr int kVTile = kVRows * kVRow;
+  static constexpr int kNBuf = (2 * (kKTile + kVTile) <= 144 * 1024) ? 2 : 1;
+  // eight waves (two per SIMD, <= 256 registers each) unless the shape needs the full register file
+  static constexpr int kNW = (kNBuf == 1 || (!k16 && D >= 128) || (k16 && D >= 256)) ? 4 : 8;
+  static constexpr int kBM = 32 * kNW;
+  static constexpr int kThreads = 64 * kNW;
   static constexpr int kQRegs = k16 ? (D / 16) * 4 : D / 2;  // dwords of Q held per lane
   static constexpr int kDB = D >= 32 ? D / 32 : 1;           // 32-wide d blocks of the output
+  static constexpr int kKLoads = kKTile / 1024;              // wave-level 1 KB DMA instructions per K tile
+  static constexpr int kVLoads = kVTile / 1024;
 };
 
-template <int AM> __device__ __forceinline__ float attn_prob(float d, float c0) {
-  if constexpr (AM == ATT_2) return fmaxf(d, 0.f);
+template <int AM> __device__ __forceinline__ float attn_prob(float r, float qs, float c0) {
+  // r = s - tau_raw in raw score units; the result only needs to be proportional to the probability
+  // (the output is normalised by the row sum), so alpha = 1.5 and 2 skip the scale.
+  if constexpr (AM == ATT_2) return fmaxf(r, 0.f);
   if constexpr (AM == ATT_15) {
-    float r = fmaxf(d, 0.f);
-    return r * r;
+    float u = fmaxf(r, 0.f);
+    return u * u;
   }
-  return d > 0.f ? fast_exp2(fast_log2(d) * c0) : 0.f;
+  return r > 0.f ? fast_exp2(fast_log2(r * qs) * c0) : 0.f;
 }
 
 template <typename T, int D, int AM>
-__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(AttnParams p) {
   using G = TileGeo<T, D>;
+  using KS = Swz<G::kKRow>;
+  using VS = Swz<G::kVRow>;
   constexpr bool k16 = G::k16;
-  extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* kbuf0 = smem;
-  unsigned char* vbuf0 = smem + G::kNBuf * G::kKTile;
-  uint32_t* maskA = reinterpret_cast<uint32_t*>(smem + G::kNBuf * (G::kKTile + G::kVTile));
-  uint32_t* maskB = maskA + kMaskWords;
+  constexpr int NW = G::kNW;
+  constexpr int BM = G::kBM;
+  // one array per pipeline stage: distinct objects let the compiler see that the DMA into one stage
+  // never aliases the ds_reads of the other
+  __shared__ __align__(1024) unsigned char k_lds0[G::kKTile];
+  __shared__ __align__(1024) unsigned char v_lds0[G::kVTile];
+  __shared__ __align__(1024) unsigned char k_lds1[G::kNBuf == 2 ? G::kKTile : 16];
+  __shared__ __align__(1024) unsigned char v_lds1[G::kNBuf == 2 ? G::kVTile : 16];
+  __shared__ uint32_t mask_a[kMaskWords];
+  __shared__ uint32_t mask_b[kMaskWords];
+  __shared__ uint32_t mask_out[2][kMaskWords];  // per 128-row half of the row block, for the bmask output
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, lq = lane & 31, lh = lane >> 5;
@@ -90,18 +121,19 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
   // Hardware block ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical
   // ids so the row blocks and grouped heads that share one K/V head hit the same L2.  Inside a K/V head
   // the longest (last) row blocks of a causal problem go first.
+  const int n_mblk = (p.N + BM - 1) / BM;
   const int group = p.Hq / p.Hkv;
-  const long long total = (long long)p.B * p.Hkv * p.n_mblk * group;
+  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
   const long long per_xcd = (total + 7) / 8;
   const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return;
   const int hg = (int)(logical % group);
-  const int mi = (int)((logical / group) % p.n_mblk);
-  const int bkv = (int)(logical / ((long long)group * p.n_mblk));
+  const int mi = (int)((logical / group) % n_mblk);
+  const int bkv = (int)(logical / ((long long)group * n_mblk));
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int h = kvh * group + hg;
-  const int mblk = p.n_mblk - 1 - mi;
-  const int m0 = mblk * kBM;
+  const int mblk = n_mblk - 1 - mi;
+  const int m0 = mblk * BM;
 
   const int N = p.N;
   int L = N;
@@ -112,26 +144,33 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
 
   const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;  // elements
   const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
-  int32_t* bmask_out = p.bmask ? p.bmask + ((size_t)(b * p.Hq + h) * p.n_mblk + mblk) * p.mask_words : nullptr;
+  // bmask rows are 128 query rows each, whatever BM this instantiation uses
+  constexpr int kHalves = BM / kMaskRows;
+  int32_t* bmask_out =
+      p.bmask ? p.bmask + ((size_t)(b * p.Hq + h) * p.n_mblk + (size_t)mblk * kHalves) * p.mask_words : nullptr;
 
   const int qi = m0 + wave * 32 + lq;  // this lane's query row
 
   // Row block entirely inside the padding: zero output rows, empty mask.
   if (m0 >= L) {
-    if (bmask_out && tid < p.mask_words) bmask_out[tid] = 0;
+    if (bmask_out) {
+      for (int i = tid; i < kHalves * p.mask_words; i += G::kThreads)
+        if (m0 + (i / p.mask_words) * kMaskRows < N) bmask_out[i] = 0;
+    }
     constexpr int kRowDw = D * G::kEB / 4;
     uint32_t* o32 = reinterpret_cast<uint32_t*>(p.out) + (qo_base + (size_t)m0 * D) * G::kEB / 4;
-    const int rows = (N - m0) < kBM ? (N - m0) : kBM;
-    for (int i = tid; i < rows * kRowDw; i += kThreads) o32[i] = 0u;
+    const int rows = (N - m0) < BM ? (N - m0) : BM;
+    for (int i = tid; i < rows * kRowDw; i += G::kThreads) o32[i] = 0u;
     return;
   }
 
-  const int row_hi = (m0 + kBM < L ? m0 + kBM : L);          // keys needed by the causal block: [0, row_hi)
+  const int row_hi = (m0 + BM < L ? m0 + BM : L);  // keys needed by the causal block: [0, row_hi)
   const int nt = p.causal ? (row_hi + kBN - 1) / kBN : (L + kBN - 1) / kBN;
   const int lim = p.causal ? (qi < L - 1 ? qi : L - 1) : L - 1;  // last valid key of this lane's row
   const int wave_row0 = m0 + wave * 32;
+  const float qs = p.qscale, inv_qs = 1.f / p.qscale;
 
-  // ---- Q fragments, pre-scaled by (alpha-1)/sqrt(D) and rounded back to the input type ----------------
+  // ---- Q fragments (unscaled) --------------------------------------------------------------------------
   uint32_t qf[G::kQRegs];
   {
     const bool ok = qi < N;
@@ -141,74 +180,55 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
       for (int ks = 0; ks < D / 16; ++ks) {
         u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float lo = unpack_lo<T>(raw[e]) * p.qscale, hi = unpack_hi<T>(raw[e]) * p.qscale;
-          qf[ks * 4 + e] = ok ? pack2<T>(lo, hi) : 0u;
-        }
+        for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = ok ? raw[e] : 0u;
       }
     } else {
       const float* qrow = reinterpret_cast<const float*>(p.q) + qo_base + (size_t)(ok ? qi : 0) * D;
 #pragma unroll
       for (int g = 0; g < D / 8; ++g) {
-        f32x4 raw = *reinterpret_cast<const f32x4*>(qrow + 8 * g + 4 * lh);
+        u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + 8 * g + 4 * lh);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) qf[g * 4 + e] = ok ? __builtin_bit_cast(uint32_t, raw[e] * p.qscale) : 0u;
+        for (int e = 0; e < 4; ++e) qf[g * 4 + e] = ok ? raw[e] : 0u;
       }
     }
   }
 
-  // ---- tile staging ---------------------------------------------------------------------------------
+  // ---- tile DMA ---------------------------------------------------------------------------------------
   const unsigned char* kglob = reinterpret_cast<const unsigned char*>(p.k) + kv_base * G::kEB;
   const unsigned char* vglob =
       k16 ? reinterpret_cast<const unsigned char*>(p.vt) + ((size_t)(b * p.Hkv + kvh) * D) * p.Npad * 2
           : reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kEB;
-  u32x4 kreg[G::kKPerThread];
-  u32x4 vreg[G::kVPerThread];
 
-  auto load_k = [&](int kt) {
+  // Wave-level load j of a tile fills LDS bytes [1024 j, 1024 j + 1024): chunk position P = 64 j + lane
+  // belongs to row P / kC, stored chunk P % kC, i.e. logical chunk (P % kC) ^ sw(row).
+  auto issue_k = [&](unsigned char* kb, int kt) {
 #pragma unroll
-    for (int i = 0; i < G::kKPerThread; ++i) {
-      int c = tid + i * kThreads;
-      int key = c / G::kKChunksPerRow, seg = c % G::kKChunksPerRow;
-      int gk = kt * kBN + key;
-      u32x4 z = {0u, 0u, 0u, 0u};
-      kreg[i] = (c < G::kKChunks && gk < N)
-                    ? *reinterpret_cast<const u32x4*>(kglob + ((size_t)gk * D) * G::kEB + seg * 16)
-                    : z;
-    }
-  };
-  auto store_k = [&](unsigned char* kb) {
-#pragma unroll
-    for (int i = 0; i < G::kKPerThread; ++i) {
-      int c = tid + i * kThreads;
-      int key = c / G::kKChunksPerRow, seg = c % G::kKChunksPerRow;
-      if (c < G::kKChunks) *reinterpret_cast<u32x4*>(kb + key * G::kKPitch + seg * 16) = kreg[i];
-    }
-  };
-  auto load_v = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < G::kVPerThread; ++i) {
-      int c = tid + i * kThreads;
-      int row = c / G::kVChunksPerRow, seg = c % G::kVChunksPerRow;
-      u32x4 z = {0u, 0u, 0u, 0u};
-      if constexpr (k16) {
-        vreg[i] = (c < G::kVChunks)
-                      ? *reinterpret_cast<const u32x4*>(vglob + ((size_t)row * p.Npad + (size_t)kt * kBN) * 2 + seg * 16)
-                      : z;
-      } else {
+    for (int j0 = 0; j0 < (G::kKLoads + NW - 1) / NW; ++j0) {
+      const int j = j0 * NW + wave;
+      if (G::kKLoads % NW == 0 || j < G::kKLoads) {
+        const int P = j * 64 + lane;
+        const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
         int gk = kt * kBN + row;
-        vreg[i] = (c < G::kVChunks && gk < N)
-                      ? *reinterpret_cast<const u32x4*>(vglob + ((size_t)gk * D) * 4 + seg * 16)
-                      : z;
+        gk = gk < N ? gk : N - 1;  // rows past the end are masked later; any valid row will do
+        dma16(kglob + (size_t)gk * G::kKRow + c * 16, kb + j * 1024);
       }
     }
   };
-  auto store_v = [&](unsigned char* vb) {
+  auto issue_v = [&](unsigned char* vb, int kt) {
 #pragma unroll
-    for (int i = 0; i < G::kVPerThread; ++i) {
-      int c = tid + i * kThreads;
-      int row = c / G::kVChunksPerRow, seg = c % G::kVChunksPerRow;
-      if (c < G::kVChunks) *reinterpret_cast<u32x4*>(vb + row * G::kVPitch + seg * 16) = vreg[i];
+    for (int j0 = 0; j0 < (G::kVLoads + NW - 1) / NW; ++j0) {
+      const int j = j0 * NW + wave;
+      if (G::kVLoads % NW == 0 || j < G::kVLoads) {
+        const int P = j * 64 + lane;
+        const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
+        if constexpr (k16) {
+          dma16(vglob + ((size_t)row * p.Npad + (size_t)kt * kBN) * 2 + c * 16, vb + j * 1024);
+        } else {
+          int gk = kt * kBN + row;
+          gk = gk < N ? gk : N - 1;  // p = 0 there
+          dma16(vglob + (size_t)gk * G::kVRow + c * 16, vb + j * 1024);
+        }
+      }
     }
   };
 
@@ -227,55 +247,70 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
     return -1;
   };
 
-  // Runs body(kt, kbuf, vbuf) over the selected tiles with the next tile's global loads in flight.
+  // Runs body(kt, k_tile, v_tile) over the selected tiles; the DMA of the next tile is issued right
+  // after the barrier that publishes the current one and completes under the current tile's MFMAs.
   auto tile_loop = [&](const uint32_t* mask, bool with_v, auto&& body) {
-    __syncthreads();  // previous pass is done with the LDS tiles and the masks are visible
+    __syncthreads();  // the previous pass is done with the LDS tiles; its mask writes are visible
     int cur = next_tile(mask, -1);
     if (cur >= 0) {
-      load_k(cur);
-      if (with_v) load_v(cur);
-      store_k(kbuf0);
-      if (with_v) store_v(vbuf0);
+      issue_k(k_lds0, cur);
+      if (with_v) issue_v(v_lds0, cur);
     }
-    __syncthreads();
-    int it = 0;
     while (cur >= 0) {
-      const int nxt = next_tile(mask, cur);
-      if (nxt >= 0) {
-        load_k(nxt);
-        if (with_v) load_v(nxt);
-      }
-      const int bi = G::kNBuf == 2 ? (it & 1) : 0;
-      body(cur, kbuf0 + bi * G::kKTile, vbuf0 + bi * G::kVTile);
-      if constexpr (G::kNBuf == 1) __syncthreads();
-      if (nxt >= 0) {
-        const int bn = G::kNBuf == 2 ? ((it + 1) & 1) : 0;
-        store_k(kbuf0 + bn * G::kKTile);
-        if (with_v) store_v(vbuf0 + bn * G::kVTile);
-      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of the tile has landed
       __syncthreads();
-      cur = nxt;
-      ++it;
+      int nxt = next_tile(mask, cur);
+      if constexpr (G::kNBuf == 2) {
+        if (nxt >= 0) {
+          issue_k(k_lds1, nxt);
+          if (with_v) issue_v(v_lds1, nxt);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      body(cur, k_lds0, v_lds0);
+      if constexpr (G::kNBuf == 1) {
+        __syncthreads();
+        if (nxt >= 0) {
+          issue_k(k_lds0, nxt);
+          if (with_v) issue_v(v_lds0, nxt);
+        }
+        cur = nxt;
+      } else {
+        cur = nxt;
+        if (cur < 0) break;
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        nxt = next_tile(mask, cur);
+        if (nxt >= 0) {
+          issue_k(k_lds0, nxt);
+          if (with_v) issue_v(v_lds0, nxt);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, k_lds1, v_lds1);
+        cur = nxt;
+      }
     }
   };
 
   // S^T block: 32 keys (kb-th half of the tile) x 32 query rows, accumulator pre-loaded with `init`.
-  auto scores = [&](const unsigned char* kb_lds, int kb, float init) -> f32x16 {
+  auto scores = [&](const unsigned char* kt_lds, int kb, float init) -> f32x16 {
     f32x16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = init;
-    const unsigned char* krow = kb_lds + (kb * 32 + lq) * G::kKPitch;
+    const int row = kb * 32 + lq;
+    const unsigned char* krow = kt_lds + row * G::kKRow;
+    const int sw = KS::sw(row);
     if constexpr (k16) {
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
-        u32x4 a = *reinterpret_cast<const u32x4*>(krow + (ks * 16 + 8 * lh) * 2);
+        u32x4 a = *reinterpret_cast<const u32x4*>(krow + (((2 * ks + lh) ^ sw) << 4));
         u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
         acc = mfma_16bit<T>(a, bq, acc);
       }
     } else {
 #pragma unroll
       for (int g = 0; g < D / 8; ++g) {
-        f32x4 a = *reinterpret_cast<const f32x4*>(krow + (8 * g + 4 * lh) * 4);
+        f32x4 a = *reinterpret_cast<const f32x4*>(krow + (((2 * g + lh) ^ sw) << 4));
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], __builtin_bit_cast(float, qf[g * 4 + e]), acc, 0, 0, 0);
@@ -290,185 +325,252 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
     for (int i = 0; i < 16; ++i) acc[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? acc[i] : -INFINITY;
   };
   // Calls f(acc, kb) for the (up to two) 32-key blocks of tile kt that this wave's rows can see.
-  auto for_blocks = [&](int kt, const unsigned char* kb_lds, float init, auto&& f) {
+  auto for_blocks = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
     if (p.causal && kt * kBN > wave_row0 + 31) return;
     const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
-      f32x16 acc = scores(kb_lds, kb, init);
+      f32x16 acc = scores(kt_lds, kb, init);
       if (need_mask) mask_block(acc, kt, kb);
       f(acc, kb);
     }
   };
+  auto mark_tile = [&](uint32_t* mask, int kt) { atomicOr(&mask[kt >> 5], 1u << (kt & 31)); };
 
-  for (int i = tid; i < 2 * kMaskWords; i += kThreads) maskA[i] = 0u;
+  for (int i = tid; i < kMaskWords; i += G::kThreads) {
+    mask_a[i] = 0u;
+    mask_b[i] = 0u;
+    mask_out[0][i] = 0u;
+    mask_out[1][i] = 0u;
+  }
 
-  // ---- pass A: row max -------------------------------------------------------------------------------
-  float m = -INFINITY;
-  tile_loop(nullptr, false, [&](int kt, const unsigned char* kb_lds, const unsigned char*) {
-    for_blocks(kt, kb_lds, 0.f, [&](const f32x16& acc, int) {
+  // ---- pass A: row max (raw units) ----------------------------------------------------------------------
+  float m_raw = -INFINITY;
+  tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
+    for_blocks(kt, kt_lds, 0.f, [&](const f32x16& acc, int) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) m = fmaxf(m, acc[i]);
+      for (int i = 0; i < 16; ++i) m_raw = fmaxf(m_raw, acc[i]);
     });
   });
-  m = fmaxf(m, __shfl_xor(m, 32, 64));
+  m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+  const float m = m_raw * qs;  // row max of z = (alpha-1) q.k / sqrt(D)
 
   // Tightest a-priori bracket: tau in [m - 1, m - n^(1 - alpha)], n = number of valid keys of the row
   // (all n equal to the max is the extreme case; adasplash/adasplash_block_mask.py:167-175).
   const float n_keys = (float)(lim + 1);
   const float hi_cap = m - fast_exp2((1.f - p.alpha) * fast_log2(n_keys));
-  Bracket br;
+  Bracket br;  // in z units
   br.lo = m - 1.f;
   br.hi = hi_cap;
   br.t = 0.5f * (br.lo + br.hi);
 
   uint32_t* mask_cur = nullptr;  // mask consumed by the next pass
-  uint32_t* mask_new = maskA;    // mask produced by the running pass
+  uint32_t* mask_new = mask_a;   // mask produced by the running pass
+  const int half = (wave * 32) / kMaskRows;  // which 128-row half of the row block this wave belongs to
 
-  // ---- pass B: histogram bracket (alpha = 1.5 or 2) ----------------------------------------------------
+  // ---- pass B: histogram bracket (alpha = 1.5 or 2) ------------------------------------------------------
   if (AM != ATT_GEN && p.use_hist) {
     const float t_shift = m - 1.f;
+    const float init = -(m_raw - inv_qs);                 // accumulator starts at -(m - 1) in raw units
+    const float c8 = (float)kAttnBins * qs * 0.9999995f;  // r * c8 in [0, 8): slot = 1 + bin, slot 0 = r < 0
     float cnt[kAttnBins];
 #pragma unroll
     for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] = 0.f;
-    unsigned long long packed = 0ull;  // eight 8-bit counters, flushed before any can overflow
+    unsigned long long packed = 0ull;  // nine 7-bit counters (slot 0 collects the discarded entries)
     int since_flush = 0;
     auto flush = [&]() {
 #pragma unroll
-      for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] += (float)((uint32_t)(packed >> (8 * bI)) & 0xffu);
+      for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] += (float)((uint32_t)(packed >> (7 * (bI + 1))) & 0x7fu);
       packed = 0ull;
       since_flush = 0;
     };
-    tile_loop(nullptr, false, [&](int kt, const unsigned char* kb_lds, const unsigned char*) {
-      bool any = false;
-      for_blocks(kt, kb_lds, -t_shift, [&](const f32x16& acc, int) {
+    tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
+      unsigned long long before = packed;
+      for_blocks(kt, kt_lds, init, [&](const f32x16& acc, int) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const float d = acc[i];  // z - (m - 1), in (-inf, 1]
-          const int bin = (int)fminf(fmaxf(d * (float)kAttnBins, 0.f), (float)(kAttnBins - 1));
-          packed += d >= 0.f ? (1ull << (8 * bin)) : 0ull;
-          any |= d >= 0.f;
+          // clamp to [0, 8.5] (one v_med3): negative and -inf entries land in slot 0, and an entry that
+          // rounding pushed above the row max of pass A stays in the top slot
+          const uint32_t slot = (uint32_t)__builtin_amdgcn_fmed3f(fmaf(acc[i], c8, 1.f), 0.f, 8.5f);
+          packed += 1ull << (slot * 7u);
         }
       });
-      if (++since_flush == 7) flush();  // <= 32 increments per tile and lane: 7 tiles stay below 255
-      if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) atomicOr(&mask_new[kt >> 5], 1u << (kt & 31));
+      // a slot above 0 moved <=> some entry of this tile is a candidate (z >= m - 1)
+      const bool any = ((packed ^ before) >> 7) != 0ull;
+      if (++since_flush == 3) flush();  // <= 32 increments per tile and lane: 3 tiles stay below 128
+      if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
     });
     flush();
 #pragma unroll
     for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] += __shfl_xor(cnt[bI], 32, 64);
     float lo = (AM == ATT_15) ? hist_bracket_alpha15<kAttnBins>(cnt, t_shift) : hist_bracket_alpha2<kAttnBins>(cnt, t_shift);
-    br.lo = fmaxf(lo, t_shift);
-    br.hi = fminf(br.lo + 1.f / (float)kAttnBins, hi_cap);
+    br.lo = fmaxf(lo - 2e-6f, t_shift);
+    br.hi = fminf(br.lo + 1.f / (float)kAttnBins + 4e-6f, hi_cap);
     br.hi = fmaxf(br.hi, br.lo);
     br.t = 0.5f * (br.lo + br.hi);
     mask_cur = mask_new;
-    mask_new = maskB;
+    mask_new = mask_b;
   }
 
-  // ---- pass C: niter safeguarded Halley / Newton steps -------------------------------------------------
+  // ---- pass C: niter safeguarded Halley / Newton steps ----------------------------------------------------
   {
     float t_prev = br.t, f_prev = 0.f;
     for (int it = 0; it < p.niter; ++it) {
-      const float t = br.t;
-      const float dl = br.lo - t;  // z > lo  <=>  (z - t) > dl
+      const float init = -br.t * inv_qs;
+      const float dl = (br.lo - br.t) * inv_qs;  // z > lo  <=>  (s - t_raw) > dl
+      const bool refine = it == p.niter - 1 || mask_cur == nullptr;
       float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-      tile_loop(mask_cur, false, [&](int kt, const unsigned char* kb_lds, const unsigned char*) {
+      int cnt_pos = 0;
+      tile_loop(mask_cur, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
         float dmax = -INFINITY;
-        for_blocks(kt, kb_lds, -t, [&](const f32x16& acc, int) {
+        for_blocks(kt, kt_lds, init, [&](const f32x16& acc, int) {
+          if (refine) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dmax = fmaxf(dmax, acc[i]);
+          }
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const float d = acc[i];
-            dmax = fmaxf(dmax, d);
+            const float r = acc[i];
             if constexpr (AM == ATT_15) {
-              const float u = fmaxf(d, 0.f);
+              const float u = fmaxf(r, 0.f);
               a0 = fmaf(u, u, a0);
               a1 += u;
-              a2 += d > 0.f ? 1.f : 0.f;
+              cnt_pos += r > 0.f;
             } else if constexpr (AM == ATT_2) {
-              a0 += fmaxf(d, 0.f);
-              a1 += d > 0.f ? 1.f : 0.f;
+              a0 += fmaxf(r, 0.f);
+              cnt_pos += r > 0.f;
             } else {
-              if (d > 0.f) {
-                const float e0 = fast_exp2(fast_log2(d) * p.c0);
-                const float r = fast_rcp(d);
-                const float e1 = e0 * r;
+              if (r > 0.f) {
+                const float uz = r * qs;
+                const float e0 = fast_exp2(fast_log2(uz) * p.c0);
+                const float rc = fast_rcp(uz);
+                const float e1 = e0 * rc;
                 a0 += e0;
                 a1 += e1;
-                a2 += e1 * r;
+                a2 += e1 * rc;
               }
             }
           }
         });
-        if (__builtin_amdgcn_ballot_w64(dmax > dl) != 0ull && lane == 0) atomicOr(&mask_new[kt >> 5], 1u << (kt & 31));
+        if (refine && __builtin_amdgcn_ballot_w64(dmax > dl) != 0ull && lane == 0) mark_tile(mask_new, kt);
       });
+      if constexpr (AM == ATT_15) {
+        a0 *= qs * qs;
+        a1 *= qs;
+        a2 = (float)cnt_pos;
+      } else if constexpr (AM == ATT_2) {
+        a0 *= qs;
+        a1 = (float)cnt_pos;
+      }
       a0 += __shfl_xor(a0, 32, 64);
       a1 += __shfl_xor(a1, 32, 64);
       a2 += __shfl_xor(a2, 32, 64);
       hybrid_step(br, a0, a1, a2, p.c0, AM != ATT_2 && p.alpha <= 1.5f, p.alpha <= 2.0f, it > 0, t_prev, f_prev);
-      // the mask just written becomes the one to read; the other array is cleared for the next pass
-      __syncthreads();
-      uint32_t* old = mask_cur;
-      mask_cur = mask_new;
-      mask_new = (mask_cur == maskA) ? maskB : maskA;
-      (void)old;
-      for (int i = tid; i < kMaskWords; i += kThreads) mask_new[i] = 0u;
+      if (refine) {
+        // the mask just written becomes the one to read; the other array is cleared for a later pass
+        __syncthreads();
+        mask_cur = mask_new;
+        mask_new = (mask_cur == mask_a) ? mask_b : mask_a;
+        for (int i = tid; i < kMaskWords; i += G::kThreads) mask_new[i] = 0u;
+      }
     }
   }
   const float tau = br.t;
 
-  // ---- pass D: out = sum_j p_j v_j / sum_j p_j over the masked tiles ------------------------------------
+  // ---- pass D: out = sum_j p_j v_j / sum_j p_j over the masked tiles --------------------------------------
   f32x16 o[G::kDB];
 #pragma unroll
   for (int db = 0; db < G::kDB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float psum = 0.f;
-  tile_loop(mask_cur, true, [&](int kt, const unsigned char* kb_lds, const unsigned char* vb_lds) {
-    for_blocks(kt, kb_lds, -tau, [&](const f32x16& acc, int kb) {
-      float pv[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        pv[i] = attn_prob<AM>(acc[i], p.c0);
-        psum += pv[i];
-      }
-      if constexpr (k16) {
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          u32x4 bp = {pack2<T>(pv[8 * s], pv[8 * s + 1]), pack2<T>(pv[8 * s + 2], pv[8 * s + 3]),
-                      pack2<T>(pv[8 * s + 4], pv[8 * s + 5]), pack2<T>(pv[8 * s + 6], pv[8 * s + 7])};
-#pragma unroll
-          for (int db = 0; db < G::kDB; ++db) {
-            const int drow = db * 32 + lq;
-            u32x4 a = {0u, 0u, 0u, 0u};
-            if (D >= 32 || drow < D)
-              a = *reinterpret_cast<const u32x4*>(vb_lds + drow * G::kVPitch + (kb * 32 + 16 * s + 8 * lh) * 2);
-            o[db] = mfma_16bit<T>(a, bp, o[db]);
-          }
-        }
-      } else {
+  unsigned active16 = 0;  // 16x16 score tiles with a non-zero probability (wave-uniform count)
+  {
+    const float init = -tau * inv_qs;
+    tile_loop(mask_cur, true, [&](int kt, const unsigned char* kt_lds, const unsigned char* vt_lds) {
+      bool tile_active = false;
+      for_blocks(kt, kt_lds, init, [&](const f32x16& acc, int kb) {
+        float pv[16];
+        float bsum = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int key = kb * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+          pv[i] = attn_prob<AM>(acc[i], qs, p.c0);
+          bsum += pv[i];
+        }
+        psum += bsum;
+        tile_active |= bsum > 0.f;
+        if (p.tile_counts) {
+          // lanes 0-15 / 32-47 hold query rows 0-15, lanes 16-31 / 48-63 rows 16-31; registers 0-7 hold
+          // keys 0-15 of the block, registers 8-15 keys 16-31.
+          bool lo = false, hi = false;
 #pragma unroll
-          for (int db = 0; db < G::kDB; ++db) {
-            const int dcol = db * 32 + lq;
-            float a = 0.f;
-            if (D >= 32 || dcol < D) a = *reinterpret_cast<const float*>(vb_lds + key * G::kVPitch + dcol * 4);
-            o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, pv[i], o[db], 0, 0, 0);
+          for (int i = 0; i < 8; ++i) {
+            lo |= pv[i] > 0.f;
+            hi |= pv[8 + i] > 0.f;
+          }
+          lo = lo && qi < L;  // padded query rows are outside the domain
+          hi = hi && qi < L;
+          const unsigned long long blo = __builtin_amdgcn_ballot_w64(lo), bhi = __builtin_amdgcn_ballot_w64(hi);
+          const unsigned long long q0 = 0x0000ffff0000ffffull, q1 = 0xffff0000ffff0000ull;
+          active16 += ((blo & q0) != 0) + ((blo & q1) != 0) + ((bhi & q0) != 0) + ((bhi & q1) != 0);
+        }
+        if constexpr (k16) {
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            u32x4 bp = {pack2<T>(pv[8 * s], pv[8 * s + 1]), pack2<T>(pv[8 * s + 2], pv[8 * s + 3]),
+                        pack2<T>(pv[8 * s + 4], pv[8 * s + 5]), pack2<T>(pv[8 * s + 6], pv[8 * s + 7])};
+#pragma unroll
+            for (int db = 0; db < G::kDB; ++db) {
+              const int drow = db * 32 + lq;
+              u32x4 a = {0u, 0u, 0u, 0u};
+              if (D >= 32 || drow < D)
+                a = *reinterpret_cast<const u32x4*>(vt_lds + VS::off(drow, kb * 4 + 2 * s + lh));
+              o[db] = mfma_16bit<T>(a, bp, o[db]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = kb * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+#pragma unroll
+            for (int db = 0; db < G::kDB; ++db) {
+              const int dcol = db * 32 + lq;
+              float a = 0.f;
+              if (D >= 32 || dcol < D)
+                a = *reinterpret_cast<const float*>(vt_lds + VS::off(key, dcol >> 2) + (dcol & 3) * 4);
+              o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, pv[i], o[db], 0, 0, 0);
+            }
           }
         }
-      }
+      });
+      // final block mask: tiles in which this 128-row half really has a non-zero probability
+      if (bmask_out && __builtin_amdgcn_ballot_w64(tile_active && qi < L) != 0ull && lane == 0)
+        mark_tile(mask_out[half], kt);
     });
-  });
+  }
   psum += __shfl_xor(psum, 32, 64);
   const float inv = psum > 0.f ? 1.f / psum : 0.f;
 
-  // ---- epilogue -------------------------------------------------------------------------------------
-  if (qi < N) {
+  // ---- epilogue: normalise, transpose through LDS, 16-byte row-contiguous stores --------------------------
+  if (tid == 0 && p.tile_counts) {  // 16x16 tiles of this row block that hold at least one valid (row, key)
+    unsigned long long dom = 0;
+    for (int r0 = m0; r0 < m0 + BM && r0 < L; r0 += 16) {
+      const int last_row = (r0 + 15 < L - 1) ? r0 + 15 : L - 1;
+      dom += p.causal ? (unsigned long long)(last_row / 16 + 1) : (unsigned long long)((L + 15) / 16);
+    }
+    atomicAdd(&p.tile_counts[0], dom);
+  }
+  if (p.tile_counts && lane == 0 && active16) atomicAdd(&p.tile_counts[1], (unsigned long long)active16);
+  if (qi < L && lh == 0 && p.taus) p.taus[(size_t)(b * p.Hq + h) * N + qi] = tau;
+
+  __syncthreads();  // every wave is done reading the tile buffers; they become the transpose scratch
+  {
+    using OS = Swz<G::kKRow>;  // a wave's 32 x D output tile uses the K-tile row format
+    unsigned char* stage_arr =
+        (wave >> 1) == 0 ? k_lds0 : ((wave >> 1) == 1 ? v_lds0 : ((wave >> 1) == 2 ? k_lds1 : v_lds1));
+    unsigned char* ot = stage_arr + (wave & 1) * (32 * G::kKRow);
     const bool live = qi < L;
-    if (live && lh == 0 && p.taus) p.taus[(size_t)(b * p.Hq + h) * N + qi] = tau;
-    unsigned char* orow = reinterpret_cast<unsigned char*>(p.out) + (qo_base + (size_t)qi * D) * G::kEB;
 #pragma unroll
     for (int db = 0; db < G::kDB; ++db) {
 #pragma unroll
@@ -478,28 +580,35 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
           float x0 = live ? o[db][4 * g] * inv : 0.f, x1 = live ? o[db][4 * g + 1] * inv : 0.f;
           float x2 = live ? o[db][4 * g + 2] * inv : 0.f, x3 = live ? o[db][4 * g + 3] * inv : 0.f;
           if constexpr (k16) {
-            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
             u32x2 w = {pack2<T>(x0, x1), pack2<T>(x2, x3)};
-            *reinterpret_cast<u32x2*>(orow + d0 * 2) = w;
+            *reinterpret_cast<u32x2*>(ot + OS::off(lq, d0 >> 3) + (d0 & 7) * 2) = w;
           } else {
             f32x4 w = {x0, x1, x2, x3};
-            *reinterpret_cast<f32x4*>(orow + d0 * 4) = w;
+            *reinterpret_cast<f32x4*>(ot + OS::off(lq, d0 >> 2)) = w;
           }
         }
       }
     }
-  }
-  __syncthreads();
-  if (bmask_out && tid < p.mask_words) {
-    uint32_t w;
-    if (mask_cur) {
-      w = tid < kMaskWords ? mask_cur[tid] : 0u;
-    } else {  // no mask was built (niter = 0 without histogram): every tile of the domain was visited
-      int first = tid * 32;
-      int cntb = nt - first;
-      w = cntb >= 32 ? 0xffffffffu : (cntb > 0 ? ((1u << cntb) - 1u) : 0u);
+    // the same wave reads back what it wrote: no block barrier needed, only the LDS counter
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    unsigned char* obase = reinterpret_cast<unsigned char*>(p.out) + (qo_base + (size_t)wave_row0 * D) * G::kEB;
+    constexpr int kChunks = 32 * OS::kC;
+#pragma unroll
+    for (int j = 0; j < (kChunks + 63) / 64; ++j) {
+      const int id = j * 64 + lane;
+      const int row = id / OS::kC, c = id % OS::kC;
+      if ((kChunks % 64 == 0 || id < kChunks) && wave_row0 + row < N) {
+        u32x4 w = *reinterpret_cast<const u32x4*>(ot + OS::off(row, c));
+        *reinterpret_cast<u32x4*>(obase + (size_t)row * G::kKRow + c * 16) = w;
+      }
     }
-    bmask_out[tid] = (int32_t)w;
+  }
+  if (bmask_out) {
+    __syncthreads();
+    for (int i = tid; i < kHalves * p.mask_words; i += G::kThreads) {
+      const int hf = i / p.mask_words, w = i % p.mask_words;
+      if (m0 + hf * kMaskRows < N) bmask_out[i] = (int32_t)mask_out[hf][w];
+    }
   }
 }
 

@@ -7,19 +7,11 @@ namespace adsp {
 template <typename T, int D, int AM> static int launch_attn_one(const AttnParams& p, hipStream_t s) {
   using G = TileGeo<T, D>;
   auto kern = attn_fwd_kernel<T, D, AM>;
-  if (G::kLdsBytes > 48 * 1024) {
-    static bool configured = false;  // per (T, D, AM) instantiation; the attribute is idempotent
-    if (!configured) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              G::kLdsBytes) != hipSuccess)
-        return 1;
-      configured = true;
-    }
-  }
   const long long group = p.Hq / p.Hkv;
-  const long long total = (long long)p.B * p.Hkv * p.n_mblk * group;
+  const long long n_mblk = (p.N + G::kBM - 1) / G::kBM;
+  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
   const long long per_xcd = (total + 7) / 8;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(kThreads), G::kLdsBytes, s, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(G::kThreads), 0, s, p);
   return 0;
 }
 

@@ -4,11 +4,10 @@
 
 namespace adsp {
 
-constexpr int kBM = 128;         // query rows per workgroup
+constexpr int kMaskRows = 128;   // query rows per row block of the bmask output
 constexpr int kBN = 64;          // keys per tile
 constexpr int kAttnBins = 8;     // histogram bins of the attention solver
 constexpr int kMaskWords = 512;  // tile-mask capacity per row block: 512 * 32 tiles * 64 keys = 1M keys
-constexpr int kThreads = 256;
 
 enum AttnAlphaMode { ATT_15 = 0, ATT_2 = 1, ATT_GEN = 2 };
 
@@ -24,7 +23,7 @@ struct AttnParams {
   int varlen_bits;
   unsigned long long* tile_counts;
   int B, Hq, Hkv, N, Npad;
-  int n_mblk;      // row blocks per (b, h)
+  int n_mblk;      // 128-row blocks per (b, h) in bmask
   int mask_words;  // int32 words per row block in bmask
   int niter;
   int causal;

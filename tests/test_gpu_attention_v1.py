@@ -1,0 +1,116 @@
+"""GPU parity of the AdaSplash-1 (block-mask) forward -- any alpha in (1, 2], causal or not, varlen --
+against the dense CPU oracle."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import adasplash_amd as A
+from adasplash_amd.adasplash_block_mask import tile_sparsity
+from oracle import exact
+from tests.gpu_util import DEV, max_err, oracle_rows_of_attention, tol_for
+
+pytestmark = pytest.mark.gpu
+
+
+def run_v1(q, k, v, **kw):
+    if kw.get("varlen") is not None:
+        kw["varlen"] = kw["varlen"].to(DEV)
+    return A.adasplash_v1(q.to(DEV), k.to(DEV), v.to(DEV), **kw)
+
+
+def test_golden_fixture(golden_dir):
+    g = np.load(golden_dir / "attn_v1_alphas.npz")
+    q, k, v = (torch.tensor(g[n]) for n in "qkv")
+    varlen = torch.tensor(g["varlen"])
+    for alpha, causal in itertools.product((1.333, 1.5, 2.0), (False, True)):
+        key = f"out_a{str(alpha).replace('.', 'p')}_{'causal' if causal else 'full'}"
+        out = run_v1(q, k, v, alpha=alpha, is_causal=causal, varlen=varlen)
+        assert max_err(out, torch.tensor(g[key])) < tol_for(torch.float32, alpha)
+        # the dispatcher sends these to the same kernel
+        out2 = A.adasplash(q.to(DEV), k.to(DEV), v.to(DEV), alpha=alpha, is_causal=causal, varlen=varlen.to(DEV),
+                           niter=10 if (alpha != 1.5 or not causal) else 10)
+        assert max_err(out2, torch.tensor(g[key])) < tol_for(torch.float32, alpha)
+
+
+def test_smoke():
+    # tests/test_adasplash.py:65-82 (varlen given as an int64 tensor)
+    torch.manual_seed(42)
+    q, k, v = (torch.randn(1, 1, 128, 32) for _ in range(3))
+    varlen = torch.tensor([96])
+    out = run_v1(q, k, v, alpha=1.5, varlen=varlen, is_causal=True)
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)) < 1e-4
+
+
+@pytest.mark.parametrize("B,H", [(1, 1), (2, 2)])
+@pytest.mark.parametrize("N", [128, 256])
+@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("alpha", [1.333, 1.5, 2.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_parameter_sweep(B, H, N, D, alpha, causal):
+    # tests/test_adasplash.py:85-114 (random varlen, fp16 and fp32)
+    torch.manual_seed(42)
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        q, k, v = (torch.randn(B, H, N, D).to(dtype) for _ in range(3))
+        varlen = torch.randint(1, N + 1, (B,))
+        out = run_v1(q, k, v, alpha=alpha, is_causal=causal, varlen=varlen)
+        want = exact.dense_entmax_attention(q, k, v, alpha, causal, varlen)
+        assert max_err(out, want) < tol_for(dtype, alpha)
+
+
+def test_zero_scores_give_the_mean_of_v():
+    # tests/test_adasplash.py:173-184
+    for n in (64, 128):
+        q = torch.zeros(1, 1, n, 64)
+        out = run_v1(q, q.clone(), torch.ones(1, 1, n, 64), alpha=1.5)
+        assert torch.allclose(out.cpu(), torch.ones(1, 1, n, 64), atol=1e-4)
+
+
+def test_padding_rows_are_exactly_zero():
+    # tests/test_adasplash.py:187-201
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(2, 1, 256, 64) for _ in range(3))
+    varlen = torch.tensor([128, 64])
+    out = run_v1(q, k, v, varlen=varlen)
+    for i in range(2):
+        assert (out[i, :, int(varlen[i]):] == 0).all()
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, False, varlen)) < 1e-4
+
+
+@pytest.mark.parametrize("seq_len", [512, 1024])
+def test_large_inputs_stay_finite(seq_len):
+    # tests/test_adasplash.py:149-170
+    torch.manual_seed(0)
+    q, k, v = ((torch.randn(2, 2, seq_len, 64) * 100).half() for _ in range(3))
+    out = run_v1(q, k, v, alpha=1.5)
+    assert torch.isfinite(out).all() and out.abs().max().item() < 1e3
+
+
+def test_high_sparsity_workload_downscaled():
+    # the block-mask benchmark workload (q, k x3, alpha = 1.333, niter = 10, non-causal) at N = 2048
+    torch.manual_seed(42)
+    q, k = ((3 * torch.randn(1, 2, 2048, 64)).to(torch.bfloat16) for _ in range(2))
+    v = torch.randn(1, 2, 2048, 64).to(torch.bfloat16)
+    out, total, active = tile_sparsity(q.to(DEV), k.to(DEV), v.to(DEV), alpha=1.333, is_causal=False, niter=10)
+    want, probs, _, _ = exact.dense_entmax_attention(q, k, v, 1.333, False, return_aux=True)
+    assert max_err(out, want) < 2e-2
+    assert total == 2 * 128 * 128
+    true_active = int((probs > 0).view(1, 2, 128, 16, 128, 16).any(5).any(3).sum())
+    assert abs(active - true_active) <= 0.02 * true_active + 2  # ties at the threshold may flip a tile
+    assert active < 0.5 * total
+
+
+def test_full_size_block_mask_workload_sampled_rows():
+    g = torch.Generator().manual_seed(42)
+    B, H, N, D = 2, 16, 16384, 64
+    q = (3 * torch.randn(B, H, N, D, generator=g)).to(torch.bfloat16)
+    k = (3 * torch.randn(B, H, N, D, generator=g)).to(torch.bfloat16)
+    v = torch.randn(B, H, N, D, generator=g).to(torch.bfloat16)
+    out = run_v1(q, k, v, alpha=1.333, is_causal=False, niter=10).cpu()
+    assert torch.isfinite(out.float()).all()
+    for b, h in ((0, 0), (1, 15)):
+        rows = [0, 127, 128, 8191, 16383]
+        want = oracle_rows_of_attention(q, k, v, b, h, rows, 1.333, False, N)
+        assert max_err(out[b, h, rows], want) < 2e-2

@@ -1,0 +1,180 @@
+"""GPU parity of the AdaSplash-2 forward (causal entmax-1.5, GQA, varlen) against the dense CPU oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+import adasplash_amd as A
+from adasplash_amd import _attention
+from oracle import exact
+from tests.gpu_util import DEV, max_err, oracle_rows_of_attention, tol_for
+
+pytestmark = pytest.mark.gpu
+
+
+def run_v2(q, k, v, niter=10, varlen=None):
+    return A.adasplash_v2(q.to(DEV), k.to(DEV), v.to(DEV), niter=niter,
+                          varlen=None if varlen is None else varlen.to(DEV))
+
+
+def test_golden_fixtures(golden_dir):
+    g = np.load(golden_dir / "attn_v2_b1h8n128d64.npz")
+    q, k, v = (torch.tensor(g[n]) for n in "qkv")
+    assert max_err(run_v2(q, k, v), torch.tensor(g["out"])) < 1e-4
+    assert max_err(A.adasplash(q.to(DEV), k.to(DEV), v.to(DEV), niter=10), torch.tensor(g["out"])) < 1e-4
+    g = np.load(golden_dir / "attn_v2_gqa_varlen.npz")
+    q, k, v = (torch.tensor(g[n]) for n in "qkv")
+    out = run_v2(q, k, v, varlen=torch.tensor(g["varlen"]))
+    assert max_err(out, torch.tensor(g["out"])) < 1e-4
+
+
+def test_smoke_fp32():
+    # tests/test_adasplash_v2.py:81-97
+    torch.manual_seed(42)
+    q, k, v = (torch.randn(1, 1, 256, 32) for _ in range(3))
+    assert max_err(run_v2(q, k, v), exact.dense_entmax_attention(q, k, v, 1.5, True)) < 1e-4
+
+
+def test_smoke_varlen_gqa():
+    # tests/test_adasplash_v2.py:100-121
+    torch.manual_seed(42)
+    q = torch.randn(1, 2, 256, 32)
+    k, v = torch.randn(1, 1, 256, 32), torch.randn(1, 1, 256, 32)
+    varlen = torch.tensor([160], dtype=torch.int32)
+    out = run_v2(q, k, v, varlen=varlen)
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)) < 1e-4
+    assert (out[:, :, 160:] == 0).all()
+
+
+@pytest.mark.parametrize("seq_len", [1024, 2048])
+def test_longer_sequences_fp32(seq_len):
+    # tests/test_adasplash_v2.py:124-144 (B=2, H=2, D=64, niter=10, 1e-4)
+    torch.manual_seed(42)
+    q, k, v = (torch.randn(2, 2, seq_len, 64) for _ in range(3))
+    assert max_err(run_v2(q, k, v), exact.dense_entmax_attention(q, k, v, 1.5, True)) < 1e-4
+
+
+@pytest.mark.parametrize("lens,n", [([65, 130], 256), ([64, 1024], 1024), ([1333, 2000], 2048), ([1, 200], 200),
+                                    ([77], 77)])
+def test_varlen_lengths_that_are_not_tile_multiples(lens, n):
+    # tests/test_adasplash_v2.py:244-321; also N itself not a power of two (allowed with varlen)
+    torch.manual_seed(42)
+    B = len(lens)
+    q, k, v = (torch.randn(B, 2, n, 64) for _ in range(3))
+    for dt in (torch.int32, torch.int64):
+        varlen = torch.tensor(lens, dtype=dt)
+        out = run_v2(q, k, v, varlen=varlen)
+        assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)) < 1e-4
+        for b, L in enumerate(lens):
+            assert (out[b, :, L:] == 0).all()
+
+
+@pytest.mark.parametrize("n_kv", [1, 2, 4, 8])
+def test_gqa_matches_repeat_interleave(n_kv):
+    # tests/test_adasplash_v2.py:324-382
+    torch.manual_seed(42)
+    q = torch.randn(2, 8, 256, 64)
+    k, v = torch.randn(2, n_kv, 256, 64), torch.randn(2, n_kv, 256, 64)
+    out = run_v2(q, k, v)
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True)) < 1e-4
+    rep = run_v2(q, k.repeat_interleave(8 // n_kv, 1).contiguous(), v.repeat_interleave(8 // n_kv, 1).contiguous())
+    assert torch.equal(out, rep)
+
+
+def test_gqa_with_varlen():
+    # tests/test_adasplash_v2.py:401-457
+    torch.manual_seed(42)
+    q = torch.randn(3, 8, 512, 64)
+    k, v = torch.randn(3, 2, 512, 64), torch.randn(3, 2, 512, 64)
+    varlen = torch.tensor([512, 300, 65], dtype=torch.int32)
+    out = run_v2(q, k, v, varlen=varlen)
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)) < 1e-4
+
+
+@pytest.mark.parametrize("head_dim", [16, 32, 64, 128, 256])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_every_head_dim_and_dtype(head_dim, dtype):
+    torch.manual_seed(head_dim)
+    q, k, v = (torch.randn(1, 2, 256, head_dim).to(dtype) for _ in range(3))
+    out = run_v2(q, k, v)
+    assert out.dtype == dtype
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True)) < tol_for(dtype)
+
+
+@pytest.mark.parametrize("niter", [0, 1, 2, 10])
+def test_bench_shapes_downscaled_bf16(niter):
+    # the two v2 benchmark workloads at sizes the oracle handles, default and larger niter
+    torch.manual_seed(42)
+    q = (torch.randn(1, 4, 1024, 64) / 8).to(torch.bfloat16)
+    k, v = (torch.randn(1, 4, 1024, 64).to(torch.bfloat16) for _ in range(2))
+    tol = 2e-2 if niter >= 1 else 0.5  # niter = 0: no refinement, tau is the midpoint of the 1/8-wide histogram bracket
+    assert max_err(run_v2(q, k, v, niter=niter), exact.dense_entmax_attention(q, k, v, 1.5, True)) < tol
+    q = torch.randn(2, 8, 1024, 128).to(torch.bfloat16)
+    k, v = (torch.randn(2, 2, 1024, 128).to(torch.bfloat16) for _ in range(2))
+    varlen = torch.tensor([1024, 300], dtype=torch.int32)
+    out = run_v2(q, k, v, niter=niter, varlen=varlen)
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)) < tol
+
+
+def test_thresholds_support_and_block_mask():
+    torch.manual_seed(1)
+    q, k, v = (torch.randn(1, 2, 512, 64) for _ in range(3))
+    q = q * 3  # sharper scores so that some tiles are really empty
+    out, taus, bmask = _attention.launch_forward(q.to(DEV), k.to(DEV), v.to(DEV), version=2, alpha=1.5,
+                                                 is_causal=True, niter=10, varlen=None)
+    _, probs, tau, scores = exact.dense_entmax_attention(q, k, v, 1.5, True, return_aux=True)
+    assert (taus.double().cpu() - tau).abs().max().item() < 1e-5
+    # identical support away from ties
+    z = 0.5 * scores
+    sup_gpu = z > taus.double().cpu()[..., None]
+    clear = (z - tau[..., None]).abs() > 1e-4
+    assert (sup_gpu == (probs > 0))[clear].all()
+    # block mask: bit (row block of 128, key tile of 64) must be set wherever a probability is non-zero
+    words = bmask.cpu().view(1, 2, 4, -1)
+    act = (probs > 0).view(1, 2, 4, 128, 8, 64).any(dim=5).any(dim=3)  # [B, H, row block, key tile]
+    bits = torch.stack([(words[..., c // 32] >> (c % 32)) & 1 for c in range(8)], dim=-1).bool()
+    assert (bits | ~act).all()
+    assert not bits[..., 0, 2:].any()  # tiles above the causal diagonal of the first row block are never set
+
+
+def test_full_size_gqa_varlen_workload_properties():
+    # the headline workload at full size: padded rows zero, finite, sampled rows against the oracle
+    g = torch.Generator().manual_seed(42)
+    B, Hq, Hkv, N, D = 8, 32, 8, 8192, 128
+    q = torch.randn(B, Hq, N, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, N, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, N, D, generator=g).to(torch.bfloat16)
+    varlen = torch.randint(N // 4, N + 1, (B,), generator=g, dtype=torch.int32)
+    out = run_v2(q, k, v, niter=1, varlen=varlen).cpu()
+    assert torch.isfinite(out.float()).all()
+    for b in range(B):
+        L = int(varlen[b])
+        assert (out[b, :, L:] == 0).all()
+    for b, h in ((0, 0), (3, 17), (7, 31)):
+        L = int(varlen[b])
+        rows = [0, 1, 63, 64, 127, 128, 1000, L // 2, L - 2, L - 1]
+        want = oracle_rows_of_attention(q, k, v, b, h, rows, 1.5, True, L)
+        assert max_err(out[b, h, rows], want) < 2e-2
+
+
+def test_full_size_mha_workload_sampled_rows():
+    g = torch.Generator().manual_seed(42)
+    B, H, N, D = 4, 16, 4096, 64
+    q = (torch.randn(B, H, N, D, generator=g) / 8).to(torch.bfloat16)
+    k = torch.randn(B, H, N, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, H, N, D, generator=g).to(torch.bfloat16)
+    out = run_v2(q, k, v, niter=1).cpu()
+    for b, h in ((0, 0), (3, 15)):
+        rows = [0, 5, 64, 129, 2047, 2048, 4000, 4095]
+        want = oracle_rows_of_attention(q, k, v, b, h, rows, 1.5, True, N)
+        assert max_err(out[b, h, rows], want) < 2e-2
+
+
+def test_v_of_ones_returns_ones_and_linearity_in_v():
+    torch.manual_seed(5)
+    q, k = torch.randn(1, 2, 512, 64), torch.randn(1, 2, 512, 64)
+    v1, v2 = torch.randn(1, 2, 512, 64), torch.randn(1, 2, 512, 64)
+    ones = run_v2(q, k, torch.ones_like(v1))
+    assert (ones.cpu() - 1).abs().max().item() < 1e-5
+    a, b, c = run_v2(q, k, v1), run_v2(q, k, v2), run_v2(q, k, v1 + v2)
+    assert (a + b - c).abs().max().item() < 1e-4

@@ -1,0 +1,172 @@
+"""Drop-in surface: names, signatures, defaults and routing of the reference package
+(adasplash/__init__.py:1-85, tests/test_public_api.py:7-50), host-side argument checks, and the C ABI."""
+
+import ctypes
+import inspect
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+import adasplash_amd
+from adasplash_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_exports_are_lazy_and_versioned():
+    assert adasplash_amd.__version__ == "0.2.0"
+    for name in ["adasplash", "adasplash_v1", "adasplash_v2", "adasplash_no_block_mask", "triton_entmax",
+                 "triton_entmax_v1", "triton_entmax_v2", "triton_sparsemax", "triton_entmax15", "adasplash2"]:
+        assert name in adasplash_amd.__all__
+        assert callable(getattr(adasplash_amd, name))
+    assert not hasattr(adasplash_amd, "entmax_attention")
+
+
+def test_signatures_and_defaults():
+    sig = inspect.signature
+    assert str(sig(adasplash_amd.adasplash)) == "(q, k, v, alpha=1.5, is_causal=True, varlen=None, niter=None)"
+    assert str(sig(adasplash_amd.adasplash_v1)) == "(q, k, v, alpha=1.5, is_causal=False, varlen=None, niter=10)"
+    assert str(sig(adasplash_amd.adasplash_v2)) == "(q, k, v, niter=1, varlen=None)"
+    assert str(sig(adasplash_amd.triton_entmax)) == "(x, alpha=1.5, n_iter=2, use_histogram=True, fast_math=False)"
+    assert str(sig(adasplash_amd.triton_entmax_v2)) == "(x, alpha=1.5, n_iter=2, use_histogram=True, fast_math=False)"
+    assert str(sig(adasplash_amd.triton_entmax_v1)) == "(x, alpha=1.5, n_iter=10, fast_math=True)"
+
+
+def test_dispatcher_is_not_shadowed_by_submodules():
+    import adasplash_amd.adasplash_v2  # noqa: F401
+    import adasplash_amd.triton_entmax_v2  # noqa: F401
+
+    assert callable(adasplash_amd.adasplash_v2) and callable(adasplash_amd.triton_entmax_v2)
+    assert list(inspect.signature(adasplash_amd.adasplash_v2).parameters) == ["q", "k", "v", "niter", "varlen"]
+
+
+def test_dispatcher_routing(monkeypatch):
+    calls = []
+    import adasplash_amd.adasplash_block_mask as v1mod
+    import adasplash_amd.adasplash_v2 as v2mod
+
+    monkeypatch.setattr(v1mod, "sparse_attn", lambda q, k, v, **kw: calls.append(("v1", kw)))
+    monkeypatch.setattr(v2mod, "sparse_attn", lambda q, k, v, **kw: calls.append(("v2", kw)))
+    adasplash_amd.adasplash(1, 2, 3)
+    adasplash_amd.adasplash(1, 2, 3, alpha=1.333)
+    adasplash_amd.adasplash(1, 2, 3, is_causal=False)
+    adasplash_amd.adasplash(1, 2, 3, niter=4)
+    adasplash_amd.adasplash(1, 2, 3, alpha=2.0, niter=3)
+    assert calls[0] == ("v2", {"niter": 1, "varlen": None})
+    assert calls[1] == ("v1", {"alpha": 1.333, "is_causal": True, "varlen": None, "niter": 10})
+    assert calls[2] == ("v1", {"alpha": 1.5, "is_causal": False, "varlen": None, "niter": 10})
+    assert calls[3] == ("v2", {"niter": 4, "varlen": None})
+    assert calls[4][0] == "v1" and calls[4][1]["niter"] == 3
+
+
+def test_entmax_argument_fixups(monkeypatch):
+    import adasplash_amd.triton_entmax_v2 as mod
+
+    seen = []
+    monkeypatch.setattr(mod._EntmaxRows, "apply", staticmethod(lambda *a: seen.append(a)))
+    mod.triton_entmax("x", alpha=1.333, n_iter=2)
+    mod.triton_entmax("x", alpha=1.5)
+    mod.triton_sparsemax("x", n_iter=5)
+    mod.triton_entmax15("x")
+    assert seen[0] == ("x", 1.333, 10, False, False)  # no histogram, at least 10 steps
+    assert seen[1] == ("x", 1.5, 2, True, False)
+    assert seen[2] == ("x", 2.0, 5, True, False)
+    assert seen[3] == ("x", 1.5, 2, True, False)
+
+
+# ---- host-side checks fire before anything touches a device (adasplash_v2.py:1248-1276) ---------------
+def _qkv(B=1, H=2, N=128, D=32, Hkv=None):
+    Hkv = H if Hkv is None else Hkv
+    return torch.zeros(B, H, N, D), torch.zeros(B, Hkv, N, D), torch.zeros(B, Hkv, N, D)
+
+
+def test_v2_rejects_bad_arguments():
+    q, k, v = _qkv(D=24)
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q, k, v)
+    q, k, v = _qkv(N=32)
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q, k, v)
+    q, k, v = _qkv(N=96)
+    with pytest.raises(AssertionError):  # not a power of two without varlen
+        adasplash_amd.adasplash_v2(q, k, v)
+    q, k, v = _qkv(H=3, Hkv=2)
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q, k, v)
+    q, k, v = _qkv()
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q.transpose(1, 2).contiguous().transpose(1, 2), k, v)
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q, k, v, varlen=torch.tensor([[128]]))
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q, k, v, varlen=torch.tensor([128.0]))
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v2(q, k, v[:, :, :64])
+
+
+def test_v1_and_entmax_reject_bad_arguments():
+    q, k, v = _qkv(N=96)
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v1(q, k, v)
+    q, k, v = _qkv(D=48)
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v1(q, k, v)
+    q, k, v = _qkv()
+    with pytest.raises(AssertionError):
+        adasplash_amd.adasplash_v1(q, k, v, varlen=torch.tensor([[1]]))
+    with pytest.raises(AssertionError):
+        adasplash_amd.triton_entmax(torch.zeros(4, 8).t())
+
+
+def test_there_is_no_cpu_fallback():
+    q, k, v = _qkv()
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        adasplash_amd.adasplash_v2(q, k, v)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        adasplash_amd.adasplash_v1(q, k, v)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        adasplash_amd.triton_entmax(torch.zeros(2, 8))
+
+
+def test_package_never_imports_the_oracle():
+    for path in (ROOT / "adasplash_amd").rglob("*.py"):
+        assert not re.search(r"^\s*(from|import)\s+oracle", path.read_text(), re.M), path
+
+
+# ---- C ABI -----------------------------------------------------------------------------------------
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "adasplash_hip.h").read_text()
+    declared = set(re.findall(r"\b(adsp_[a-z0-9_]+)\s*\(", header))
+    assert {"adsp_entmax_rows_fwd", "adsp_attn_v2_fwd", "adsp_attn_v1_fwd", "adsp_attn_workspace_bytes"} <= declared
+    lib = ctypes.CDLL(str(_lib.lib_path()))
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/adasplash_hip.h but not exported"
+
+
+def test_sizing_helpers_and_status_strings():
+    lib = _lib.load()
+    assert lib.adsp_version() >= 1
+    assert lib.adsp_attn_workspace_bytes(8, 8, 8192, 128, _lib.ADSP_BF16) == 8 * 8 * 128 * 8192 * 2
+    assert lib.adsp_attn_workspace_bytes(2, 2, 100, 64, _lib.ADSP_F16) == 2 * 2 * 64 * 128 * 2  # keys padded to 64
+    assert lib.adsp_attn_workspace_bytes(8, 8, 8192, 128, _lib.ADSP_F32) == 0
+    assert lib.adsp_attn_bmask_words(8192) == 64 * 4 and lib.adsp_attn_bmask_words(64) == 1
+    assert lib.adsp_status_string(0) == b"ok"
+    assert all(len(lib.adsp_status_string(s)) > 0 for s in range(0, 9))
+
+
+def test_argument_errors_come_back_as_status_codes():
+    lib = _lib.load()
+    # no pointer is dereferenced and nothing is launched for these
+    assert lib.adsp_entmax_rows_fwd(None, None, 4, 8, 0, 1.5, 2, 1, 0, None) == 1
+    assert lib.adsp_entmax_rows_fwd(None, None, 0, 8, 0, 1.5, 2, 1, 0, None) == 0
+    assert lib.adsp_entmax_rows_fwd(16, 16, 4, 8, 9, 1.5, 2, 1, 0, None) == 3
+    assert lib.adsp_entmax_rows_fwd(16, 16, 4, 8, 0, 1.0, 2, 1, 0, None) == 5
+    assert lib.adsp_attn_v2_fwd(None, None, None, None, None, None, None, 0, 1, 1, 1, 64, 64, 1, 1, None, 0, None) == 1
+    assert lib.adsp_attn_v2_fwd(16, 16, 16, 16, None, None, None, 0, 1, 3, 2, 64, 64, 1, 1, None, 0, None) == 2
+    assert lib.adsp_attn_v2_fwd(16, 16, 16, 16, None, None, None, 0, 1, 1, 1, 64, 48, 1, 1, None, 0, None) == 2
+    assert lib.adsp_attn_v2_fwd(16, 16, 16, 8, None, None, None, 0, 1, 1, 1, 64, 64, 1, 1, None, 0, None) == 4
+    assert lib.adsp_attn_v2_fwd(16, 16, 16, 16, None, None, None, 0, 1, 1, 1, 64, 64, 1, 1, None, 0, None) == 6
+    assert lib.adsp_attn_v1_fwd(16, 16, 16, 16, None, None, None, 0, 1, 1, 64, 64, 0, 2.5, 0, 1, None, 0, None,
+                                None) == 5
