@@ -9,8 +9,10 @@ int launch_attn_bf16(const AttnParams& p, int D, int am, hipStream_t s);
 int launch_attn_f16(const AttnParams& p, int D, int am, hipStream_t s);
 int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s);
 
-// Key-major, MFMA-ordered copy of V for the 16-bit path:
-//   vt[bh, d, pos(n)] = v[bh, n, d],  pos(16s + 8a + 4h + r) = 16s + 8h + 4a + r,  zero for n >= N.
+// Tile-wise key-major, MFMA-ordered copy of V for the 16-bit path.  Keys are cut in tiles of 64; a tile
+// is stored as one contiguous [D][64] block (so the kernel fetches it with contiguous kilobyte copies):
+//   vt[bh, kt, d, pos(n % 64)] = v[bh, n, d],  kt = n / 64,
+//   pos(16s + 8a + 4h + r) = 16s + 8h + 4a + r,  zero for n >= N.
 // With this order a lane of the PV product reads its 8 keys {16s + 4h + r, 16s + 8 + 4h + r} of one
 // d row as one 16-byte LDS access.
 __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
@@ -27,14 +29,13 @@ __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restri
     tile[key * pitch + d] = gk < N ? vsrc[(size_t)gk * D + d] : (uint16_t)0;
   }
   __syncthreads();
-  uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64;
+  uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64 * D;
   for (int i = threadIdx.x; i < 64 * D; i += 256) {
     int d = i / 64, pos = i % 64;
     int key = (pos & ~15) | (((pos >> 2) & 1) << 3) | (((pos >> 3) & 1) << 2) | (pos & 3);
-    vdst[(size_t)d * Npad + pos] = tile[key * pitch + d];
+    vdst[i] = tile[key * pitch + d];
   }
 }
-
 
 static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
 static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }

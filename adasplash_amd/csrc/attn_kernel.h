@@ -22,7 +22,7 @@
 //   D  p = [z - tau]_+^c0, out += P V over masked tiles, divided by sum p at the end.
 // The accumulator of the S^T MFMA is initialised with -tau (resp. -(m-1)), so z - tau costs no VALU op.
 //
-// The 16-bit path consumes V through a key-major copy (vt_layout_kernel) so that the PV product
+// The 16-bit path consumes V through a tile-wise key-major copy (vt_layout_kernel) so that the PV product
 // out^T = V^T P^T can take P^T straight from the S^T accumulators without an LDS round trip.
 #pragma once
 #include "common.h"
@@ -88,9 +88,9 @@ template <typename T, int D> struct TileGeo {
 template <int AM> __device__ __forceinline__ float attn_prob(float r, float qs, float c0) {
   // r = s - tau_raw in raw score units; the result only needs to be proportional to the probability
   // (the output is normalised by the row sum), so alpha = 1.5 and 2 skip the scale.
-  if constexpr (AM == ATT_2) return fmaxf(r, 0.f);
+  if constexpr (AM == ATT_2) return __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
   if constexpr (AM == ATT_15) {
-    float u = fmaxf(r, 0.f);
+    float u = __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
     return u * u;
   }
   return r > 0.f ? fast_exp2(fast_log2(r * qs) * c0) : 0.f;
@@ -115,7 +115,8 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
   __shared__ uint32_t mask_out[2][kMaskWords];  // per 128-row half of the row block, for the bmask output
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+  const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
 
   // ---- XCD-aware block -> (batch, kv head, row block, head in group) mapping -------------------------
   // Hardware block ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical
@@ -222,7 +223,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
         const int P = j * 64 + lane;
         const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
         if constexpr (k16) {
-          dma16(vglob + ((size_t)row * p.Npad + (size_t)kt * kBN) * 2 + c * 16, vb + j * 1024);
+          dma16(vglob + (size_t)kt * G::kVTile + row * G::kVRow + c * 16, vb + j * 1024);
         } else {
           int gk = kt * kBN + row;
           gk = gk < N ? gk : N - 1;  // p = 0 there
@@ -292,8 +293,50 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
     }
   };
 
-  // S^T block: 32 keys (kb-th half of the tile) x 32 query rows, accumulator pre-loaded with `init`.
-  auto scores = [&](const unsigned char* kt_lds, int kb, float init) -> f32x16 {
+  // S^T of one tile: two 32-key blocks x 32 query rows, accumulators pre-loaded with `init`.  The K
+  // fragments of a block are fetched together so that its MFMA chain can run back to back, and the two
+  // chains are independent, which lets the second one cover the first one's result latency.
+  auto tile_scores = [&](const unsigned char* kt_lds, float init, f32x16& s0, f32x16& s1) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s0[i] = init;
+      s1[i] = init;
+    }
+    const unsigned char* krow0 = kt_lds + lq * G::kKRow;
+    const unsigned char* krow1 = kt_lds + (32 + lq) * G::kKRow;
+    const int sw0 = KS::sw(lq), sw1 = KS::sw(32 + lq);
+    if constexpr (k16) {
+      u32x4 a0[D / 16], a1[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a0[ks] = *reinterpret_cast<const u32x4*>(krow0 + (((2 * ks + lh) ^ sw0) << 4));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a1[ks] = *reinterpret_cast<const u32x4*>(krow1 + (((2 * ks + lh) ^ sw1) << 4));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s0 = mfma_16bit<T>(a0[ks], bq, s0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s1 = mfma_16bit<T>(a1[ks], bq, s1);
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < D / 8; ++g) {
+        f32x4 a0 = *reinterpret_cast<const f32x4*>(krow0 + (((2 * g + lh) ^ sw0) << 4));
+        f32x4 a1 = *reinterpret_cast<const f32x4*>(krow1 + (((2 * g + lh) ^ sw1) << 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float bq = __builtin_bit_cast(float, qf[g * 4 + e]);
+          s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[e], bq, s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[e], bq, s1, 0, 0, 0);
+        }
+      }
+    }
+  };
+  // S^T of one 32-key block of the tile (used where register pressure forbids holding both blocks).
+  auto block_scores = [&](const unsigned char* kt_lds, int kb, float init) -> f32x16 {
     f32x16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = init;
@@ -301,11 +344,13 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
     const unsigned char* krow = kt_lds + row * G::kKRow;
     const int sw = KS::sw(row);
     if constexpr (k16) {
+      u32x4 a[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(krow + (((2 * ks + lh) ^ sw) << 4));
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
-        u32x4 a = *reinterpret_cast<const u32x4*>(krow + (((2 * ks + lh) ^ sw) << 4));
         u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
-        acc = mfma_16bit<T>(a, bq, acc);
+        acc = mfma_16bit<T>(a[ks], bq, acc);
       }
     } else {
 #pragma unroll
@@ -324,14 +369,31 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? acc[i] : -INFINITY;
   };
-  // Calls f(acc, kb) for the (up to two) 32-key blocks of tile kt that this wave's rows can see.
-  auto for_blocks = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
+  // Calls f(s0, s1) with the two score blocks of tile kt unless no row of this wave can see the tile.
+  // Tiles that touch the causal diagonal or the sequence tail take the masked instantiation; both are
+  // straight-line code so MFMA, LDS and VALU work of the two blocks can be interleaved.
+  auto for_tile = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
+    if (p.causal && kt * kBN > wave_row0 + 31) return;
+    const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
+    f32x16 s0, s1;
+    if (need_mask) {
+      tile_scores(kt_lds, init, s0, s1);
+      mask_block(s0, kt, 0);
+      mask_block(s1, kt, 1);
+      f(s0, s1);
+    } else {
+      tile_scores(kt_lds, init, s0, s1);
+      f(s0, s1);
+    }
+  };
+  // Block-by-block variant: f(s, kb) per visible 32-key block.
+  auto for_tile_blocks = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
     if (p.causal && kt * kBN > wave_row0 + 31) return;
     const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
-      f32x16 acc = scores(kt_lds, kb, init);
+      f32x16 acc = block_scores(kt_lds, kb, init);
       if (need_mask) mask_block(acc, kt, kb);
       f(acc, kb);
     }
@@ -348,9 +410,9 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
   // ---- pass A: row max (raw units) ----------------------------------------------------------------------
   float m_raw = -INFINITY;
   tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
-    for_blocks(kt, kt_lds, 0.f, [&](const f32x16& acc, int) {
+    for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) m_raw = fmaxf(m_raw, acc[i]);
+      for (int i = 0; i < 16; ++i) m_raw = fmaxf(fmaxf(m_raw, s0[i]), s1[i]);
     });
   });
   m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
@@ -371,13 +433,22 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
 
   // ---- pass B: histogram bracket (alpha = 1.5 or 2) ------------------------------------------------------
   if (AM != ATT_GEN && p.use_hist) {
-    const float t_shift = m - 1.f;
-    const float init = -(m_raw - inv_qs);                 // accumulator starts at -(m - 1) in raw units
-    const float c8 = (float)kAttnBins * qs * 0.9999995f;  // r * c8 in [0, 8): slot = 1 + bin, slot 0 = r < 0
+    // Bins are laid on z - t_shift with t_shift a hair below m - 1, so that the rounding differences
+    // between this pass and pass A cannot push the row maximum out of the top bin.
+    const float margin = 1.f / 4096.f;                       // in z units
+    const float t_shift = m - 1.f - margin;
+    const float init = -(m_raw - (1.f + margin) * inv_qs);  // accumulator starts at -t_shift in raw units
+    // the bins span [0, 1 + 2 margin) above t_shift, which puts the maximum (at 1 + margin) inside the top one
+    const float span = 1.f + 2.f * margin;
+    const float c8 = (float)kAttnBins * qs / span;
+    const float bin_w = span / (float)kAttnBins;  // bin width in z units
     float cnt[kAttnBins];
 #pragma unroll
     for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] = 0.f;
-    unsigned long long packed = 0ull;  // nine 7-bit counters (slot 0 collects the discarded entries)
+    // Nine 7-bit counters in one 64-bit register: slot 0 collects the discarded entries (r < 0; the
+    // float -> uint conversion saturates them to 0), slot 1 + b counts bin b.  An entry that rounding
+    // still lifted past the top edge would shift into bit 63, which nothing reads.
+    unsigned long long packed = 0ull;
     int since_flush = 0;
     auto flush = [&]() {
 #pragma unroll
@@ -387,16 +458,15 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
     };
     tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
       unsigned long long before = packed;
-      for_blocks(kt, kt_lds, init, [&](const f32x16& acc, int) {
+      for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          // clamp to [0, 8.5] (one v_med3): negative and -inf entries land in slot 0, and an entry that
-          // rounding pushed above the row max of pass A stays in the top slot
-          const uint32_t slot = (uint32_t)__builtin_amdgcn_fmed3f(fmaf(acc[i], c8, 1.f), 0.f, 8.5f);
-          packed += 1ull << (slot * 7u);
+        for (int i = 0; i < 32; ++i) {
+          const float r = i < 16 ? s0[i & 15] : s1[i & 15];
+          const uint32_t slot = (uint32_t)fmaf(r, c8, 1.f);
+          packed += 1ull << __umul24(slot, 7u);
         }
       });
-      // a slot above 0 moved <=> some entry of this tile is a candidate (z >= m - 1)
+      // a slot above 0 moved <=> some entry of this tile is a candidate (z >= t_shift)
       const bool any = ((packed ^ before) >> 7) != 0ull;
       if (++since_flush == 3) flush();  // <= 32 increments per tile and lane: 3 tiles stay below 128
       if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
@@ -404,10 +474,12 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
     flush();
 #pragma unroll
     for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] += __shfl_xor(cnt[bI], 32, 64);
-    float lo = (AM == ATT_15) ? hist_bracket_alpha15<kAttnBins>(cnt, t_shift) : hist_bracket_alpha2<kAttnBins>(cnt, t_shift);
-    br.lo = fmaxf(lo - 2e-6f, t_shift);
-    br.hi = fminf(br.lo + 1.f / (float)kAttnBins + 4e-6f, hi_cap);
-    br.hi = fmaxf(br.hi, br.lo);
+    // Every entry counts as sitting on the lower edge of its bin (the maximum included), which gives a
+    // lower bound lo of tau with tau <= lo + bin width whenever no entry was lost.  The upper end is used
+    // for the starting point only; the bracket keeps the unconditional bound hi_cap.
+    float lo = (AM == ATT_15) ? hist_bracket_alpha15<kAttnBins>(cnt, t_shift, bin_w) : hist_bracket_alpha2<kAttnBins>(cnt, t_shift, bin_w);
+    br.lo = fmaxf(lo - 2e-6f, m - 1.f);
+    br.hi = fminf(br.lo + bin_w + 4e-6f, hi_cap);
     br.t = 0.5f * (br.lo + br.hi);
     mask_cur = mask_new;
     mask_new = mask_b;
@@ -424,21 +496,21 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
       int cnt_pos = 0;
       tile_loop(mask_cur, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
         float dmax = -INFINITY;
-        for_blocks(kt, kt_lds, init, [&](const f32x16& acc, int) {
+        for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
           if (refine) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) dmax = fmaxf(dmax, acc[i]);
+            for (int i = 0; i < 16; ++i) dmax = fmaxf(fmaxf(dmax, s0[i]), s1[i]);
           }
 #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float r = acc[i];
+          for (int i = 0; i < 32; ++i) {
+            const float r = i < 16 ? s0[i & 15] : s1[i & 15];
             if constexpr (AM == ATT_15) {
-              const float u = fmaxf(r, 0.f);
+              const float u = __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
               a0 = fmaf(u, u, a0);
               a1 += u;
               cnt_pos += r > 0.f;
             } else if constexpr (AM == ATT_2) {
-              a0 += fmaxf(r, 0.f);
+              a0 += __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
               cnt_pos += r > 0.f;
             } else {
               if (r > 0.f) {
@@ -466,6 +538,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
       a0 += __shfl_xor(a0, 32, 64);
       a1 += __shfl_xor(a1, 32, 64);
       a2 += __shfl_xor(a2, 32, 64);
+      // f is convex and decreasing, so a Newton step from the left never passes the root: if it lands
+      // beyond the upper end although f(t) > 0, that end (the histogram's lo + bin width) was not valid
+      // for this row and the unconditional bound takes its place.
+      if (a0 > 1.f && br.t + (a0 - 1.f) / (p.c0 * a1) > br.hi) br.hi = hi_cap;
       hybrid_step(br, a0, a1, a2, p.c0, AM != ATT_2 && p.alpha <= 1.5f, p.alpha <= 2.0f, it > 0, t_prev, f_prev);
       if (refine) {
         // the mask just written becomes the one to read; the other array is cleared for a later pass
@@ -490,7 +566,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
     const float init = -tau * inv_qs;
     tile_loop(mask_cur, true, [&](int kt, const unsigned char* kt_lds, const unsigned char* vt_lds) {
       bool tile_active = false;
-      for_blocks(kt, kt_lds, init, [&](const f32x16& acc, int kb) {
+      for_tile_blocks(kt, kt_lds, init, [&](const f32x16& acc, int kb) {
         float pv[16];
         float bsum = 0.f;
 #pragma unroll

@@ -115,7 +115,8 @@ __device__ __forceinline__ float solve_row(const Row& row, const RowsParams& p, 
       }
     });
     row_sum<TPR, kRowBins>(cnt, sm);
-    br.lo = (AM == AM_15) ? hist_bracket_alpha15<kRowBins>(cnt, t_shift) : hist_bracket_alpha2<kRowBins>(cnt, t_shift);
+    br.lo = (AM == AM_15) ? hist_bracket_alpha15<kRowBins>(cnt, t_shift, 1.f / kRowBins, true, 1.f)
+                          : hist_bracket_alpha2<kRowBins>(cnt, t_shift, 1.f / kRowBins, true, 1.f);
     br.lo = fmaxf(br.lo, t_shift);
     br.hi = fminf(br.lo + 1.f / (float)kRowBins, m);
     br.t = hist_start_point<kRowBins>(cnt, t_shift, br.lo, br.hi);

@@ -6,41 +6,48 @@
 
 namespace adsp {
 
-// Lower bracket from a histogram of z - (max - 1) on [0, 1] split in BINS equal bins, alpha = 1.5.
-// Every member of a bin is placed on the bin's lower edge, the bins are taken greedily from the top
-// while the quantised threshold stays below the bin edge, and the threshold of the accepted set has
-// the closed form below.  The maximum itself enters as the unit element (count - 1 in the top bin).
-// Follows adasplash/adasplash_v2.py:434-461 and adasplash/triton_entmax_v2.py:135-155.
+// Lower bound of tau from a histogram of z - t_shift on BINS bins of width w starting at 0, alpha = 1.5.
+// Every member of a bin is placed on the bin's lower edge e, the bins are taken greedily from the top
+// while the quantised threshold stays below the bin edge (n e^2 - 2 e sum z + sum z^2 < 1), and the
+// threshold of the accepted set has the closed form below.  Since quantising scores downwards by at most
+// w moves tau downwards by at most w, the result lo satisfies lo <= tau <= lo + w.
+// With `exact_max` the row maximum, known to sit at max_pos above t_shift, enters with its exact value
+// instead of its bin edge (the reference's variant: adasplash/adasplash_v2.py:434-461,
+// adasplash/triton_entmax_v2.py:135-155, where max_pos = 1 and w = 1 / BINS).
 template <int BINS>
-__device__ __forceinline__ float hist_bracket_alpha15(const float (&cnt)[BINS], float t_shift) {
-  float sz = 1.f, sk = 1.f, szz = 1.f;
+__device__ __forceinline__ float hist_bracket_alpha15(const float (&cnt)[BINS], float t_shift, float w = 1.f / (float)BINS,
+                                                      bool exact_max = false, float max_pos = 1.f) {
+  float sz = exact_max ? max_pos : 0.f, sk = exact_max ? 1.f : 0.f, szz = exact_max ? max_pos * max_pos : 0.f;
 #pragma unroll
   for (int sj = BINS - 1; sj >= 0; --sj) {
-    float c = cnt[sj] - (sj == BINS - 1 ? 1.f : 0.f);
-    const float e = (float)sj / (float)BINS;
+    float c = cnt[sj] - ((exact_max && sj == BINS - 1) ? 1.f : 0.f);
+    const float e = (float)sj * w;
     float nz = sz + c * e, nk = sk + c, nzz = szz + c * (e * e);
     bool good = nk * e * e - 2.f * nz * e + nzz < 1.f;
     sz = good ? nz : sz;
     sk = good ? nk : sk;
     szz = good ? nzz : szz;
   }
+  sk = fmaxf(sk, 1.f);
   float disc = fmaxf(sz * sz - sk * (szz - 1.f), 0.f);
   return t_shift + (sz - sqrtf(disc)) / sk;
 }
 
-// Same for alpha = 2 (adasplash/triton_entmax_v2.py:114-131).
+// Same for alpha = 2 (adasplash/triton_entmax_v2.py:114-131): accept while sum z - n e < 1.
 template <int BINS>
-__device__ __forceinline__ float hist_bracket_alpha2(const float (&cnt)[BINS], float t_shift) {
-  float sz = 1.f, sk = 1.f;
+__device__ __forceinline__ float hist_bracket_alpha2(const float (&cnt)[BINS], float t_shift, float w = 1.f / (float)BINS,
+                                                     bool exact_max = false, float max_pos = 1.f) {
+  float sz = exact_max ? max_pos : 0.f, sk = exact_max ? 1.f : 0.f;
 #pragma unroll
   for (int sj = BINS - 1; sj >= 0; --sj) {
-    float c = cnt[sj] - (sj == BINS - 1 ? 1.f : 0.f);
-    const float e = (float)sj / (float)BINS;
+    float c = cnt[sj] - ((exact_max && sj == BINS - 1) ? 1.f : 0.f);
+    const float e = (float)sj * w;
     float nz = sz + c * e, nk = sk + c;
     bool good = (nz - nk * e) < 1.f;
     sz = good ? nz : sz;
     sk = good ? nk : sk;
   }
+  sk = fmaxf(sk, 1.f);
   return t_shift + (sz - 1.f) / sk;
 }
 
