@@ -11,9 +11,9 @@ struct bf16_t { uint16_t bits; };  // storage-only tags; arithmetic is always fp
 struct f16_t { uint16_t bits; };
 
 template <typename T> struct elem_traits;
-template <> struct elem_traits<float> { static constexpr int kBytes = 4; static constexpr int kVec = 4; };
-template <> struct elem_traits<bf16_t> { static constexpr int kBytes = 2; static constexpr int kVec = 8; };
-template <> struct elem_traits<f16_t> { static constexpr int kBytes = 2; static constexpr int kVec = 8; };
+template <> struct elem_traits<float> { static constexpr int kBytes = 4; static constexpr int kVec = 4; static constexpr bool kIsBf16 = false; };
+template <> struct elem_traits<bf16_t> { static constexpr int kBytes = 2; static constexpr int kVec = 8; static constexpr bool kIsBf16 = true; };
+template <> struct elem_traits<f16_t> { static constexpr int kBytes = 2; static constexpr int kVec = 8; static constexpr bool kIsBf16 = false; };
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
 __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {

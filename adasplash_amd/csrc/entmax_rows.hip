@@ -141,80 +141,6 @@ __device__ __forceinline__ float solve_row(const Row& row, const RowsParams& p, 
   return br.t;
 }
 
-// ---- register-resident rows ------------------------------------------------------------------------
-template <typename T, int NCHUNK, int TPR> struct RegRow {
-  static constexpr int kVec = elem_traits<T>::kVec;
-  float z[NCHUNK * kVec];
-  template <typename F> __device__ __forceinline__ void for_each(F f) const {
-#pragma unroll
-    for (int i = 0; i < NCHUNK * kVec; ++i) f(z[i]);
-  }
-};
-
-template <typename T, int AM, int NCHUNK, int TPR>
-__global__ __launch_bounds__(256) void entmax_rows_reg_kernel(RowsParams p) {
-  constexpr int kVec = elem_traits<T>::kVec;
-  constexpr int kRowsPerBlock = 256 / TPR;
-  __shared__ float sm[32];
-  const int tid = threadIdx.x;
-  const int t_in_row = tid % TPR;
-  long long row = (long long)blockIdx.x * kRowsPerBlock + tid / TPR;
-  // TPR == 256: one row per block, every thread is active.  TPR == 64: a wave owns a row, and a wave
-  // past the last row simply leaves (no block-level barrier is used in that configuration).
-  if (row >= p.rows) return;
-
-  const long long nvec = p.cols / kVec;
-  const u32x4* xrow = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.x) +
-                                                     (size_t)row * p.cols * elem_traits<T>::kBytes);
-  u32x4* yrow = reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.y) + (size_t)row * p.cols * elem_traits<T>::kBytes);
-
-  RegRow<T, NCHUNK, TPR> r;
-  u32x4 raw[NCHUNK];
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c) {
-    long long vi = (long long)c * TPR + t_in_row;
-    if (vi < nvec) raw[c] = __builtin_nontemporal_load(xrow + vi);
-  }
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c) {
-    long long vi = (long long)c * TPR + t_in_row;
-    const bool ok = vi < nvec;
-    const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
-    if constexpr (kVec == 4) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) r.z[c * 4 + e] = ok ? __builtin_bit_cast(float, w[e]) * p.scale : -INFINITY;
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        r.z[c * 8 + 2 * e] = ok ? unpack_lo<T>(w[e]) * p.scale : -INFINITY;
-        r.z[c * 8 + 2 * e + 1] = ok ? unpack_hi<T>(w[e]) * p.scale : -INFINITY;
-      }
-    }
-  }
-
-  const float tau = solve_row<AM, TPR>(r, p, sm);
-
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c) {
-    long long vi = (long long)c * TPR + t_in_row;
-    if (vi < nvec) {
-      u32x4 o;
-      if constexpr (kVec == 4) {
-        o.x = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 0] - tau, p.c0));
-        o.y = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 1] - tau, p.c0));
-        o.z = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 2] - tau, p.c0));
-        o.w = __builtin_bit_cast(uint32_t, prob<AM>(r.z[c * 4 + 3] - tau, p.c0));
-      } else {
-        o.x = pack2<T>(prob<AM>(r.z[c * 8 + 0] - tau, p.c0), prob<AM>(r.z[c * 8 + 1] - tau, p.c0));
-        o.y = pack2<T>(prob<AM>(r.z[c * 8 + 2] - tau, p.c0), prob<AM>(r.z[c * 8 + 3] - tau, p.c0));
-        o.z = pack2<T>(prob<AM>(r.z[c * 8 + 4] - tau, p.c0), prob<AM>(r.z[c * 8 + 5] - tau, p.c0));
-        o.w = pack2<T>(prob<AM>(r.z[c * 8 + 6] - tau, p.c0), prob<AM>(r.z[c * 8 + 7] - tau, p.c0));
-      }
-      __builtin_nontemporal_store(o, yrow + vi);
-    }
-  }
-}
-
 // ---- streaming rows (any length / alignment): one 256-thread block per row, scalar accesses --------
 template <typename T> __device__ __forceinline__ float load_elem(const void* base, size_t i);
 template <> __device__ __forceinline__ float load_elem<float>(const void* b, size_t i) { return ((const float*)b)[i]; }
@@ -233,20 +159,181 @@ template <> __device__ __forceinline__ void store_elem<f16_t>(void* b, size_t i,
   ((uint16_t*)b)[i] = (uint16_t)float_to_f16_bits(v);
 }
 
-template <typename T> struct StreamRow {
+template <typename T, int TPR> struct StreamRow {
   const void* x;
   size_t base;
   long long cols;
   float scale;
+  int t_in_row;
   template <typename F> __device__ __forceinline__ void for_each(F f) const {
-    for (long long j = threadIdx.x; j < cols; j += 256) f(load_elem<T>(x, base + j) * scale);
+    for (long long j = t_in_row; j < cols; j += TPR) f(load_elem<T>(x, base + j) * scale);
   }
 };
+
+// ---- register-resident rows ------------------------------------------------------------------------
+// The row stays in registers as loaded (raw 16-byte chunks).  Only entries with z >= max - 1 can be in the
+// support (tau >= max - 1 for every alpha), so after the max pass those candidates are compacted into a
+// short LDS list and the whole threshold solve runs on that list inside one wave; the other entries are
+// touched twice more at most: one compare against the candidate threshold and one against tau, both
+// done per 16-byte chunk on the chunk's maximum.  Rows with more candidates than the list holds fall
+// back to solving on the full register copy.
+constexpr int kCandPerLane = 16;
+constexpr int kCandCap = 64 * kCandPerLane;  // list capacity per row
+
+template <typename T> __device__ __forceinline__ float chunk_elem(u32x4 raw, int e) {
+  // the element is copied to a scalar first: bit-casting a vector-element expression directly makes this
+  // compiler read element 0 whatever the index
+  if constexpr (elem_traits<T>::kVec == 4) {
+    const uint32_t w = raw[e];
+    return __builtin_bit_cast(float, w);
+  } else {
+    const uint32_t w = raw[e >> 1];
+    return (e & 1) ? unpack_hi<T>(w) : unpack_lo<T>(w);
+  }
+}
+
+template <int K> struct ListRow {
+  float z[K];
+  template <typename F> __device__ __forceinline__ void for_each(F f) const {
+#pragma unroll
+    for (int i = 0; i < K; ++i) f(z[i]);
+  }
+  __device__ __forceinline__ void load(const float* list, int n, int lane) {
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      const int idx = i * 64 + lane;
+      z[i] = idx < n ? list[idx] : -INFINITY;
+    }
+  }
+};
+
+// Register budget: rows of up to 16 chunks per lane are compiled for four waves per SIMD (128 registers),
+// except fp16 whose unpacking needs more live values; longer rows get two waves (256 registers).
+template <typename T, int NCHUNK> constexpr int rows_min_waves() {
+  return (NCHUNK <= 8 || (NCHUNK <= 16 && (elem_traits<T>::kVec == 4 || elem_traits<T>::kIsBf16))) ? 4 : 2;
+}
+
+template <typename T, int AM, int NCHUNK, int TPR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(rows_min_waves<T, NCHUNK>()))) void entmax_rows_reg_kernel(RowsParams p) {
+  constexpr int kVec = elem_traits<T>::kVec;
+  constexpr int kRowsPerBlock = 256 / TPR;
+  __shared__ float sm[32];
+  __shared__ float cand[kRowsPerBlock][kCandCap];
+  __shared__ int cand_n[kRowsPerBlock];
+  const int tid = threadIdx.x;
+  const int t_in_row = tid % TPR, r_in_blk = tid / TPR, lane = tid & 63;
+  long long row = (long long)blockIdx.x * kRowsPerBlock + r_in_blk;
+  // TPR == 256: one row per block, every thread is active.  TPR == 64: a wave owns a row, and a wave
+  // past the last row simply leaves (no block-level barrier is used in that configuration).
+  if (row >= p.rows) return;
+
+  const long long nvec = p.cols / kVec;
+  const u32x4* xrow = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.x) +
+                                                     (size_t)row * p.cols * elem_traits<T>::kBytes);
+  u32x4* yrow = reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.y) + (size_t)row * p.cols * elem_traits<T>::kBytes);
+
+  struct {
+    u32x4 raw[NCHUNK];
+    bool valid[NCHUNK];
+  } r;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    long long vi = (long long)c * TPR + t_in_row;
+    r.valid[c] = vi < nvec;
+    if (r.valid[c]) r.raw[c] = __builtin_nontemporal_load(xrow + vi);
+  }
+  if (t_in_row == 0) cand_n[r_in_blk] = 0;
+
+  // pass 1: per-chunk and row maxima, in the input's own units
+  float cmax[NCHUNK];
+  float xm = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    float cm = -INFINITY;
+    if constexpr (kVec == 4) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) cm = fmaxf(cm, chunk_elem<T>(r.raw[c], e));
+    } else if constexpr (sizeof(T) == 2 && elem_traits<T>::kIsBf16) {
+      // bf16: the upper element of a dword is compared as the dword itself (the lower element only adds
+      // mantissa bits below one bf16 ulp), so a chunk maximum may exceed the true one by less than an
+      // ulp -- harmless for the two "can this chunk matter" tests, and removed from the row maximum below
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t w = r.raw[c][e];
+        cm = fmaxf(cm, fmaxf(__builtin_bit_cast(float, w), __builtin_bit_cast(float, w << 16)));
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) cm = fmaxf(cm, chunk_elem<T>(r.raw[c], e));
+    }
+    cmax[c] = r.valid[c] ? cm : -INFINITY;
+    xm = fmaxf(xm, cmax[c]);
+  }
+  xm = row_max<TPR>(xm, sm);  // (TPR == 256: its barriers also publish cand_n = 0)
+  if constexpr (elem_traits<T>::kIsBf16) xm = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, xm) & 0xffff0000u);
+
+  // pass 2: compact the candidates z >= max - 1 into the row's LDS list
+  const float x_thr = xm - p.c0;  // (alpha-1) x >= (alpha-1) xm - 1
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    if (cmax[c] >= x_thr) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const float x = chunk_elem<T>(r.raw[c], e);
+        if (x >= x_thr) {
+          const int idx = atomicAdd(&cand_n[r_in_blk], 1);
+          if (idx < kCandCap) cand[r_in_blk][idx] = x * p.scale;
+        }
+      }
+    }
+  }
+  if constexpr (TPR > 64) __syncthreads();
+  const int n_cand = cand_n[r_in_blk];
+
+  float tau;
+  if (n_cand <= 64) {
+    // every wave of the row solves the same short list redundantly: wave-level reductions only.  The
+    // usual case (a peaked row) has at most one candidate per lane.
+    ListRow<1> lr;
+    lr.load(cand[r_in_blk], n_cand, lane);
+    tau = solve_row<AM, 64>(lr, p, sm);
+  } else if (n_cand <= kCandCap) {
+    ListRow<kCandPerLane> lr;
+    lr.load(cand[r_in_blk], n_cand, lane);
+    tau = solve_row<AM, 64>(lr, p, sm);
+  } else {
+    // too many candidates for the list: solve on the whole row, re-read (from L2) pass by pass
+    StreamRow<T, TPR> sr{p.x, (size_t)row * p.cols, p.cols, p.scale, t_in_row};
+    tau = solve_row<AM, TPR>(sr, p, sm);
+  }
+
+  // pass 3: outputs; a chunk whose maximum is not above tau is all zeros
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    if (r.valid[c]) {
+      long long vi = (long long)c * TPR + t_in_row;
+      u32x4 o = {0u, 0u, 0u, 0u};
+      if (cmax[c] * p.scale > tau) {
+        if constexpr (kVec == 4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = __builtin_bit_cast(uint32_t, prob<AM>(chunk_elem<T>(r.raw[c], e) * p.scale - tau, p.c0));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = pack2<T>(prob<AM>(chunk_elem<T>(r.raw[c], 2 * e) * p.scale - tau, p.c0),
+                            prob<AM>(chunk_elem<T>(r.raw[c], 2 * e + 1) * p.scale - tau, p.c0));
+        }
+      }
+      __builtin_nontemporal_store(o, yrow + vi);
+    }
+  }
+}
 
 template <typename T, int AM> __global__ __launch_bounds__(256) void entmax_rows_stream_kernel(RowsParams p) {
   __shared__ float sm[32];
   for (long long row = blockIdx.x; row < p.rows; row += gridDim.x) {
-    StreamRow<T> r{p.x, (size_t)row * p.cols, p.cols, p.scale};
+    StreamRow<T, 256> r{p.x, (size_t)row * p.cols, p.cols, p.scale, (int)threadIdx.x};
     const float tau = solve_row<AM, 256>(r, p, sm);
     for (long long j = threadIdx.x; j < p.cols; j += 256) {
       float z = load_elem<T>(p.x, r.base + j) * p.scale;
@@ -296,8 +383,9 @@ template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool a
   const bool can_reg = aligned && (p.cols % kVec == 0) && p.rows < (1ll << 31);
   if (can_reg) {
     const long long c64 = (nvec + 63) / 64, c256 = (nvec + 255) / 256;
-    // A wave per row while the row fits in <= 64 registers per lane; four waves per row beyond that.
-    int tpr = (c64 * kVec <= 64) ? 64 : 256;
+    // A wave per row (no block barriers) while the row fits in 16 16-byte chunks per lane (128 registers
+    // keep four waves per SIMD resident); four waves per row beyond that.
+    int tpr = c64 <= 16 ? 64 : 256;
     if (force_tpr == 64 && c64 <= 32) tpr = 64;
     if (force_tpr == 256) tpr = 256;
     if (tpr == 64) {
