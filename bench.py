@@ -28,6 +28,11 @@ import torch
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these
+# same workloads, each counter scaled by what it reads for a plain 1 GiB copy (FETCH_SIZE x 2.0,
+# WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
+MEASURED_HBM_TRAFFIC_BYTES = {"c4": 1.243e9, "c3": None, "c5": None, "c2_f32": 1.0739e9, "c2_bf16": 0.5373e9}
+
 
 def _events_ms(fn, steps, warmup):
     for _ in range(warmup):
@@ -168,7 +173,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy"])
     ap.add_argument("--no-extra", action="store_true", help="skip the entmax-rows and CPU-baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -184,20 +189,31 @@ def main():
     line = {"metric": "v2 fwd ms + eff. TFLOPS/%MFMA peak (N=8192,D=128,GQA); entmax rows GB/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "data": "synthetic"}
+    if args.workload == "copy":
+        # plain device copy of known size: the reference point for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE
+        x = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_(0, 255)
+        y = torch.empty_like(x)
+        ms, _ = _events_ms(lambda: y.copy_(x), args.steps, args.warmup)
+        line.update({"value": 2 * x.numel() / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "dtype": "u8",
+                     "config": {"workload": "copy: torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)"}})
+        print(json.dumps(line))
+        return
     if args.workload == "c2":
         rows = bench_rows(args.steps, args.warmup, device)
         best = rows["f32_alpha1.5"]
         line.update({"value": best["GBps"], "unit": "GB/s", "ms_per_step": best["ms"], "dtype": "f32",
                      "config": {"workload": "c2: entmax rows [16384, 8192] fp32 alpha=1.5, hist init, n_iter=2"},
                      "roofline": {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                  "frac": best["frac_hbm_peak"], "traffic": None},
+                                  "frac": best["frac_hbm_peak"], "traffic": MEASURED_HBM_TRAFFIC_BYTES["c2_f32"],
+                                  "kernel": "entmax_rows_reg_kernel", "bytes_per_launch": best["bytes"]},
                      "extra": {"entmax_rows": rows}})
     else:
         res = bench_attention(args.workload, args.steps, args.warmup, device)
         line.update({"value": res["eff_tflops"], "unit": "TFLOP/s", "ms_per_step": res["ms_per_step"],
                      "dtype": "bf16", "config": res["config"],
                      "roofline": {"bound": "mfma", "achieved": res["eff_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                                  "unit": "TFLOP/s", "frac": res["frac_mfma_peak"], "traffic": None,
+                                  "unit": "TFLOP/s", "frac": res["frac_mfma_peak"],
+                                  "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
                                   "kernel": "attn_fwd_kernel", "flops_per_launch": res["flops_per_step"]},
                      "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k == "wall_ms_per_step"}})
         if not args.no_extra:
