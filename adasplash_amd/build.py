@@ -30,7 +30,8 @@ FLAGS = [
 
 # The attention kernels never produce or consume NaNs on purpose (masked scores are -inf and are clamped
 # before any product), so fmax/fmin need no sNaN-quieting pre-pass there.
-EXTRA_FLAGS = {"attn_bf16": ["-fno-honor-nans"], "attn_f16": ["-fno-honor-nans"], "attn_f32": ["-fno-honor-nans"]}
+_ATTN_FLAGS = ["-fno-honor-nans"] + os.environ.get("ADSP_ATTN_FLAGS", "").split()
+EXTRA_FLAGS = {"attn_bf16": _ATTN_FLAGS, "attn_f16": _ATTN_FLAGS, "attn_f32": _ATTN_FLAGS}
 
 
 def _compile(src: Path) -> Path:
