@@ -50,11 +50,33 @@ def assert_contiguous(*inputs, msg="Inputs are not contiguous."):
     assert all(t.is_contiguous() for t in inputs), msg
 
 
-_BACKWARD_MSG = (
-    "the MI355X build implements the forward pass of sparse entmax attention only; "
-    "the backward kernels are not built yet"
-)
+def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
+    """Enqueue the dQ and dK/dV kernels on the current stream; returns ``(dq, dk, dv)``.
 
-
-def backward_not_built():
-    raise NotImplementedError(_BACKWARD_MSG)
+    ``taus`` / ``bmask`` are the thresholds and the tile mask the forward produced.  Rows of ``dout`` past a
+    sequence's valid length are ignored (zeroed here, as the reference's masked loads do,
+    adasplash/adasplash_v2.py:1030-1033).
+    """
+    _lib.require_device(q, k, v, dout, varlen)
+    lib = _lib.load()
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    dt = _lib.dtype_code(q)
+    dout = dout.to(q.dtype).contiguous()
+    if varlen is not None:
+        valid = torch.arange(N, device=q.device)[None, :] < varlen.to(torch.long)[:, None]
+        dout = dout * valid[:, None, :, None].to(dout.dtype)
+    dq = torch.empty_like(q)
+    dk = torch.empty_like(k)
+    dv = torch.empty_like(v)
+    delta = torch.empty((B, Hq, N), device=q.device, dtype=torch.float32)
+    zinv = torch.empty((B, Hq, N), device=q.device, dtype=torch.float32)
+    ws_bytes = lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dt)
+    ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
+    with torch.cuda.device(q.device):
+        st = lib.adsp_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), taus.data_ptr(),
+                               _lib.ptr(bmask), _lib.ptr(varlen), _varlen_bits(varlen), dq.data_ptr(), dk.data_ptr(),
+                               dv.data_ptr(), delta.data_ptr(), zinv.data_ptr(), B, Hq, Hkv, N, D, dt, float(alpha),
+                               int(bool(is_causal)), _lib.ptr(ws), ws_bytes, _lib.current_stream(q.device))
+        _lib.check(st, "adsp_attn_bwd")
+    return dq, dk, dv

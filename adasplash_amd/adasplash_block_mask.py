@@ -31,11 +31,17 @@ class _SparseAttentionV1(torch.autograd.Function):
         )
         ctx.save_for_backward(q, k, v, taus, bmask)
         ctx.alpha = alpha
+        ctx.is_causal = is_causal
+        ctx.varlen = varlen
         return out
 
     @staticmethod
     def backward(ctx, do):
-        _attention.backward_not_built()
+        q, k, v, taus, bmask = ctx.saved_tensors
+        dq, dk, dv = _attention.launch_backward(
+            q, k, v, do, taus, bmask, alpha=ctx.alpha, is_causal=ctx.is_causal, varlen=ctx.varlen
+        )
+        return dq, dk, dv, None, None, None, None
 
 
 def sparse_attn(q, k, v, alpha=1.5, is_causal=False, varlen=None, niter=10):

@@ -44,7 +44,11 @@ class _SparseAttentionV2(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do):
-        _attention.backward_not_built()
+        q, k, v, taus, bmask = ctx.saved_tensors
+        dq, dk, dv = _attention.launch_backward(
+            q, k, v, do, taus, bmask, alpha=1.5, is_causal=True, varlen=ctx.varlen
+        )
+        return dq, dk, dv, None, None
 
 
 def sparse_attn(q, k, v, niter=1, varlen=None):

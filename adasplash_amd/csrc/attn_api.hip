@@ -1,6 +1,7 @@
-// C ABI of the attention forward: argument checks, V re-layout launch, kernel dispatch.
+// C ABI of the attention forward and backward: argument checks, re-layout launches, kernel dispatch.
 #include "common.h"
 #include "attn_params.h"
+#include "attn_bwd_params.h"
 #include <math.h>
 #include "../../include/adasplash_hip.h"
 
@@ -8,6 +9,9 @@ namespace adsp {
 int launch_attn_bf16(const AttnParams& p, int D, int am, hipStream_t s);
 int launch_attn_f16(const AttnParams& p, int D, int am, hipStream_t s);
 int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s);
+int launch_attn_bwd_bf16(const AttnBwdParams& p, int D, int am, hipStream_t s);
+int launch_attn_bwd_f16(const AttnBwdParams& p, int D, int am, hipStream_t s);
+int launch_attn_bwd_f32(const AttnBwdParams& p, int D, int am, hipStream_t s);
 
 // Tile-wise key-major, MFMA-ordered copy of V for the 16-bit path.  Keys are cut in tiles of 64; a tile
 // is stored as one contiguous [D][64] block (so the kernel fetches it with contiguous kilobyte copies):
@@ -119,6 +123,79 @@ extern "C" int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, voi
   if (alpha > 2.0) return ADSP_ERR_UNSUPPORTED;
   return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, H, H, N, D, dtype, alpha, is_causal, niter,
                            0, workspace, workspace_bytes, tile_counts, (hipStream_t)stream);
+}
+
+extern "C" size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype) {
+  if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
+  return (size_t)B * (Hkv + 2 * (size_t)Hq) * D * adsp::npad_of(N) * 2;
+}
+
+extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* taus,
+                             const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
+                             float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
+                             int is_causal, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace adsp;
+  hipStream_t s = (hipStream_t)stream;
+  if (!q || !k || !v || !dout || !taus || !dq || !dk || !dv || !delta || !zinv) return ADSP_ERR_NULL;
+  if (dtype != ADSP_F32 && dtype != ADSP_BF16 && dtype != ADSP_F16) return ADSP_ERR_DTYPE;
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || Hq % Hkv != 0) return ADSP_ERR_SHAPE;
+  if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return ADSP_ERR_SHAPE;
+  if (mask_words_of(N) > kMaskWords) return ADSP_ERR_SHAPE;
+  if (!(alpha > 1.0) || alpha > 2.0) return ADSP_ERR_UNSUPPORTED;
+  if (varlen && varlen_bits != 32 && varlen_bits != 64) return ADSP_ERR_UNSUPPORTED;
+  if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)dout | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) & 15) != 0)
+    return ADSP_ERR_ALIGN;
+
+  AttnBwdParams p;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.dout = dout;
+  p.kt = p.qt = p.dot = nullptr;
+  p.dq = dq;
+  p.dk = dk;
+  p.dv = dv;
+  p.taus = taus;
+  p.delta = delta;
+  p.zinv = zinv;
+  p.bmask = bmask;
+  p.varlen = varlen;
+  p.varlen_bits = varlen_bits;
+  p.B = B;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.N = N;
+  p.Npad = npad_of(N);
+  p.n_mblk = mblocks_of(N);
+  p.mask_words = mask_words_of(N);
+  p.causal = is_causal ? 1 : 0;
+  p.qscale = (float)((alpha - 1.0) / sqrt((double)D));
+  p.sm_scale = (float)(1.0 / sqrt((double)D));
+  p.c0 = (float)(1.0 / (alpha - 1.0));
+  const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
+
+  (void)hipGetLastError();
+  if (dtype != ADSP_F32) {
+    const size_t need = adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dtype);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
+    uint16_t* kt = (uint16_t*)workspace;
+    uint16_t* qt = kt + (size_t)B * Hkv * D * p.Npad;
+    uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
+    const size_t shm = (size_t)64 * (D + 2) * 2;
+    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hkv)), dim3(256), shm, s,
+                       (const uint16_t*)k, kt, N, p.Npad, D);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hq)), dim3(256), shm, s,
+                       (const uint16_t*)q, qt, N, p.Npad, D);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hq)), dim3(256), shm, s,
+                       (const uint16_t*)dout, dot, N, p.Npad, D);
+    p.kt = kt;
+    p.qt = qt;
+    p.dot = dot;
+  }
+  int rc = dtype == ADSP_BF16 ? launch_attn_bwd_bf16(p, D, am, s)
+                              : (dtype == ADSP_F16 ? launch_attn_bwd_f16(p, D, am, s) : launch_attn_bwd_f32(p, D, am, s));
+  if (rc != 0) return ADSP_ERR_LAUNCH;
+  return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
 }
 
 extern "C" int adsp_version(void) { return 1; }

@@ -1,0 +1,618 @@
+// Backward of the sparse entmax attention for gfx950: dQ kernel and dK/dV kernel.
+//
+// With x_ij = q_i.k_j / sqrt(D), z = (alpha-1) x, p_ij = [z_ij - tau_i]_+^(1/(alpha-1)) and u = p^(2-alpha),
+// the entmax Jacobian is diag(u) - u u^T / sum(u), hence for dP_ij = dO_i . v_j
+//   delta_i = sum_j u_ij dP_ij / sum_j u_ij,   dX_ij = u_ij (dP_ij - delta_i),
+//   dQ_i = sum_j dX_ij k_j / sqrt(D),  dK_j = sum_i dX_ij q_i / sqrt(D),  dV_j = sum_i p_ij dO_i
+// (adasplash/adasplash_v2.py:839-1234 for alpha = 1.5, adasplash/adasplash_block_mask.py:493-919 for any alpha).
+// The forward divides its output by sum_j p_ij, so dV uses p_ij / sum_j p_ij as well.
+//
+// Both kernels recompute the scores with MFMA in the forward's layout: the product is taken as
+// (LDS tile rows) x (register fragments of the lane's own row), so a lane owns one query row in the dQ
+// kernel and one key row in the dK/dV kernel, and the other index runs over its 16 accumulator registers.
+//   dQ kernel, one workgroup per 128 query rows:  pass 1 accumulates sum p, sum u, sum u dP -> delta;
+//                                                 pass 2 forms dX and dQ^T += K^T dX^T.
+//   dK/dV kernel, one workgroup per 128 keys, all query heads of the K/V head in turn:
+//                                                 pass 1 dV^T += dO^T P, pass 2 dK^T += Q^T dX.
+// The 16-bit path takes the transposed operands (K^T, dO^T, Q^T) from tile-wise transposed copies in the
+// layout of vt_layout_kernel, so that P / dX go from the accumulators straight into the next MFMA.
+#pragma once
+#include "attn_kernel.h"
+#include "attn_bwd_params.h"
+
+namespace adsp {
+
+constexpr int kBwdRows = 128;  // rows (queries resp. keys) per workgroup = 4 waves x 32
+
+// p and u = p^(2-alpha) from r = z - tau.
+template <int AM> __device__ __forceinline__ void bwd_prob(float r, float c0, float& pr, float& u) {
+  if constexpr (AM == ATT_15) {
+    u = __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
+    pr = u * u;
+  } else if constexpr (AM == ATT_2) {
+    pr = __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
+    u = r > 0.f ? 1.f : 0.f;
+  } else {
+    const bool pos = r > 0.f;
+    const float rr = pos ? r : 1.f;
+    const float e = fast_exp2(fast_log2(rr) * c0);
+    pr = pos ? e : 0.f;
+    u = pos ? e * fast_rcp(rr) : 0.f;
+  }
+}
+
+template <typename T, int D> struct BwdTiles {
+  using G = TileGeo<T, D>;
+  using KS = Swz<G::kKRow>;
+  using VS = Swz<G::kVRow>;
+  static constexpr bool k16 = G::k16;
+  static constexpr int kTile = G::kKTile;  // bytes of a [64][D] tile, in either orientation
+  static constexpr int kNW = kBwdRows / 32;
+  static constexpr int kSlots = k16 ? 3 : 2;  // tiles per pipeline stage
+  static constexpr int kNBuf = (2 * kSlots * kTile <= 144 * 1024) ? 2 : 1;
+  static constexpr int kLoads = kTile / 1024;
+
+  // DMA of rows [row0, row0 + 64) of a row-major [N][D] tensor into a swizzled tile.
+  static __device__ __forceinline__ void issue_rows(const unsigned char* g, int row0, int N, unsigned char* lds, int wave,
+                                                    int lane) {
+#pragma unroll
+    for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
+      const int j = j0 * kNW + wave;
+      if (kLoads % kNW == 0 || j < kLoads) {
+        const int P = j * 64 + lane;
+        const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
+        int gr = row0 + row;
+        gr = gr < N ? gr : N - 1;  // rows past the end are masked by the caller
+        dma16(g + (size_t)gr * G::kKRow + c * 16, lds + j * 1024);
+      }
+    }
+  }
+  // DMA of one contiguous transposed tile ([D][64], as written by vt_layout_kernel) into a swizzled tile.
+  static __device__ __forceinline__ void issue_t(const unsigned char* gtile, unsigned char* lds, int wave, int lane) {
+#pragma unroll
+    for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
+      const int j = j0 * kNW + wave;
+      if (kLoads % kNW == 0 || j < kLoads) {
+        const int P = j * 64 + lane;
+        const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
+        dma16(gtile + row * G::kVRow + c * 16, lds + j * 1024);
+      }
+    }
+  }
+  // Fragments of the lane's own row (B operand of the score-like products).
+  static __device__ __forceinline__ void load_row_frags(const void* base, size_t row, bool ok, int lh,
+                                                        uint32_t (&f)[G::kQRegs]) {
+    if constexpr (k16) {
+      const uint16_t* r = reinterpret_cast<const uint16_t*>(base) + row * D;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 raw = *reinterpret_cast<const u32x4*>(r + ks * 16 + 8 * lh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[ks * 4 + e] = ok ? raw[e] : 0u;
+      }
+    } else {
+      const float* r = reinterpret_cast<const float*>(base) + row * D;
+#pragma unroll
+      for (int g = 0; g < D / 8; ++g) {
+        u32x4 raw = *reinterpret_cast<const u32x4*>(r + 8 * g + 4 * lh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[g * 4 + e] = ok ? raw[e] : 0u;
+      }
+    }
+  }
+  // acc[i] = (tile row kb*32 + 8(i/4) + 4 lh + i%4) . (lane's row), for the 32 lane rows of the wave.
+  static __device__ __forceinline__ f32x16 dot_block(const unsigned char* tile, int kb, const uint32_t (&f)[G::kQRegs],
+                                                     int lq, int lh) {
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    const int row = kb * 32 + lq;
+    const unsigned char* trow = tile + row * G::kKRow;
+    const int sw = KS::sw(row);
+    if constexpr (k16) {
+      u32x4 a[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(trow + (((2 * ks + lh) ^ sw) << 4));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 b = {f[ks * 4], f[ks * 4 + 1], f[ks * 4 + 2], f[ks * 4 + 3]};
+        acc = mfma_16bit<T>(a[ks], b, acc);
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < D / 8; ++g) {
+        f32x4 a = *reinterpret_cast<const f32x4*>(trow + (((2 * g + lh) ^ sw) << 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], __builtin_bit_cast(float, f[g * 4 + e]), acc, 0, 0, 0);
+      }
+    }
+    return acc;
+  }
+  // o^T[d][lane row] += sum over the 32 tile rows of block kb of  tile[row][d] * w[row][lane row], where
+  // w holds the lane's 16 values in the accumulator order of dot_block.  16-bit: `tile` is the transposed
+  // tile; fp32: the row-major one.
+  static __device__ __forceinline__ void acc_block(f32x16 (&o)[G::kDB], const unsigned char* tile, int kb,
+                                                   const float (&w)[16], int lq, int lh) {
+    if constexpr (k16) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        u32x4 b = {pack2<T>(w[8 * s], w[8 * s + 1]), pack2<T>(w[8 * s + 2], w[8 * s + 3]),
+                   pack2<T>(w[8 * s + 4], w[8 * s + 5]), pack2<T>(w[8 * s + 6], w[8 * s + 7])};
+#pragma unroll
+        for (int db = 0; db < G::kDB; ++db) {
+          const int drow = db * 32 + lq;
+          u32x4 a = {0u, 0u, 0u, 0u};
+          if (D >= 32 || drow < D) a = *reinterpret_cast<const u32x4*>(tile + VS::off(drow, kb * 4 + 2 * s + lh));
+          o[db] = mfma_16bit<T>(a, b, o[db]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = kb * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+#pragma unroll
+        for (int db = 0; db < G::kDB; ++db) {
+          const int dcol = db * 32 + lq;
+          float a = 0.f;
+          if (D >= 32 || dcol < D) a = *reinterpret_cast<const float*>(tile + KS::off(row, dcol >> 2) + (dcol & 3) * 4);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, w[i], o[db], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // Writes scale * o^T (32 rows of this wave x D) to rows [row0, row0 + 32) of a row-major tensor, through
+  // an LDS transpose in `stage` (32 * kKRow bytes, private to the wave).
+  static __device__ __forceinline__ void store_rows(const f32x16 (&o)[G::kDB], float scale, unsigned char* stage,
+                                                    void* gbase, int row0, int N, int lane) {
+    const int lq = lane & 31, lh = lane >> 5;
+#pragma unroll
+    for (int db = 0; db < G::kDB; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d0 = db * 32 + 8 * g + 4 * lh;
+        if (D >= 32 || d0 < D) {
+          const float x0 = o[db][4 * g] * scale, x1 = o[db][4 * g + 1] * scale;
+          const float x2 = o[db][4 * g + 2] * scale, x3 = o[db][4 * g + 3] * scale;
+          if constexpr (k16) {
+            u32x2 w = {pack2<T>(x0, x1), pack2<T>(x2, x3)};
+            *reinterpret_cast<u32x2*>(stage + KS::off(lq, d0 >> 3) + (d0 & 7) * 2) = w;
+          } else {
+            f32x4 w = {x0, x1, x2, x3};
+            *reinterpret_cast<f32x4*>(stage + KS::off(lq, d0 >> 2)) = w;
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave reads back what it wrote itself
+    unsigned char* obase = reinterpret_cast<unsigned char*>(gbase) + (size_t)row0 * G::kKRow;
+    constexpr int kChunks = 32 * KS::kC;
+#pragma unroll
+    for (int j = 0; j < (kChunks + 63) / 64; ++j) {
+      const int id = j * 64 + lane;
+      const int row = id / KS::kC, c = id % KS::kC;
+      if ((kChunks % 64 == 0 || id < kChunks) && row0 + row < N) {
+        u32x4 w = *reinterpret_cast<const u32x4*>(stage + KS::off(row, c));
+        *reinterpret_cast<u32x4*>(obase + (size_t)row * G::kKRow + c * 16) = w;
+      }
+    }
+  }
+};
+
+__device__ __forceinline__ int bwd_seq_len(const AttnBwdParams& p, int b) {
+  int L = p.N;
+  if (p.varlen) {
+    long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
+    L = (int)(l < 0 ? 0 : (l > p.N ? p.N : l));
+  }
+  return L;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dQ kernel: grid (row blocks of 128 queries, B * Hq)
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int D, int AM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void attn_bwd_dq_kernel(AttnBwdParams p) {
+  using BT = BwdTiles<T, D>;
+  using G = TileGeo<T, D>;
+  constexpr bool k16 = G::k16;
+  __shared__ __align__(1024) unsigned char a0[BT::kTile];  // K tile, row-major
+  __shared__ __align__(1024) unsigned char b0[BT::kTile];  // V tile, row-major
+  __shared__ __align__(1024) unsigned char c0[k16 ? BT::kTile : 16];  // K^T tile (16-bit)
+  __shared__ __align__(1024) unsigned char a1[BT::kNBuf == 2 ? BT::kTile : 16];
+  __shared__ __align__(1024) unsigned char b1[BT::kNBuf == 2 ? BT::kTile : 16];
+  __shared__ __align__(1024) unsigned char c1[(k16 && BT::kNBuf == 2) ? BT::kTile : 16];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+  const int N = p.N;
+  const int n_blk = (N + kBwdRows - 1) / kBwdRows;
+  const int mblk = n_blk - 1 - (int)blockIdx.x;  // the longest causal rows first
+  const int bh = blockIdx.y;
+  const int b = bh / p.Hq, h = bh % p.Hq;
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int L = bwd_seq_len(p, b);
+  const int m0 = mblk * kBwdRows;
+  const int wave_row0 = m0 + wave * 32;
+  const int qi = wave_row0 + lq;
+  const size_t q_base = (size_t)bh * N;                   // rows
+  const size_t kv_base = (size_t)(b * p.Hkv + kvh) * N;  // rows
+  unsigned char* dq_rows = reinterpret_cast<unsigned char*>(p.dq) + q_base * G::kKRow;
+
+  if (m0 >= L) {  // padding rows: zero gradient
+    constexpr int kRowDw = D * G::kEB / 4;
+    uint32_t* o32 = reinterpret_cast<uint32_t*>(dq_rows) + (size_t)m0 * kRowDw;
+    const int rows = (N - m0) < kBwdRows ? (N - m0) : kBwdRows;
+    for (int i = tid; i < rows * kRowDw; i += 256) o32[i] = 0u;
+    return;
+  }
+
+  uint32_t qf[G::kQRegs], dof[G::kQRegs];
+  {
+    const bool ok = qi < N;
+    BT::load_row_frags(p.q, q_base + (ok ? qi : 0), ok, lh, qf);
+    BT::load_row_frags(p.dout, q_base + (ok ? qi : 0), ok, lh, dof);
+  }
+  const bool live = qi < L;
+  const float tau = live ? p.taus[q_base + qi] : INFINITY;
+  const int lim = p.causal ? (qi < L - 1 ? qi : L - 1) : L - 1;  // last valid key of the lane's row
+  const int row_hi = (m0 + kBwdRows < L ? m0 + kBwdRows : L);
+  const int nt = p.causal ? (row_hi + kBN - 1) / kBN : (L + kBN - 1) / kBN;
+  const int32_t* mrow = p.bmask ? p.bmask + ((size_t)bh * p.n_mblk + mblk) * p.mask_words : nullptr;
+
+  const unsigned char* kg = reinterpret_cast<const unsigned char*>(p.k) + kv_base * G::kKRow;
+  const unsigned char* vg = reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kKRow;
+  const unsigned char* ktg =
+      k16 ? reinterpret_cast<const unsigned char*>(p.kt) + (size_t)(b * p.Hkv + kvh) * D * p.Npad * 2 : nullptr;
+
+  auto next_tile = [&](int cur) -> int {
+    int t = cur + 1;
+    if (!mrow) return t < nt ? t : -1;
+    while (t < nt) {
+      uint32_t w = (uint32_t)mrow[t >> 5] >> (t & 31);
+      if (w) {
+        t += __builtin_ctz(w);
+        return t < nt ? t : -1;
+      }
+      t = (t | 31) + 1;
+    }
+    return -1;
+  };
+  auto issue = [&](unsigned char* a, unsigned char* bb, unsigned char* c, int kt, bool with_t) {
+    BT::issue_rows(kg, kt * kBN, N, a, wave, lane);
+    BT::issue_rows(vg, kt * kBN, N, bb, wave, lane);
+    if constexpr (k16) {
+      if (with_t) BT::issue_t(ktg + (size_t)kt * BT::kTile, c, wave, lane);
+    }
+  };
+  auto tile_loop = [&](bool with_t, auto&& body) {
+    __syncthreads();
+    int cur = next_tile(-1);
+    if (cur >= 0) issue(a0, b0, c0, cur, with_t);
+    while (cur >= 0) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      int nxt = next_tile(cur);
+      if constexpr (BT::kNBuf == 2) {
+        if (nxt >= 0) issue(a1, b1, c1, nxt, with_t);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      body(cur, a0, b0, c0);
+      if constexpr (BT::kNBuf == 1) {
+        __syncthreads();
+        if (nxt >= 0) issue(a0, b0, c0, nxt, with_t);
+        cur = nxt;
+      } else {
+        cur = nxt;
+        if (cur < 0) break;
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        nxt = next_tile(cur);
+        if (nxt >= 0) issue(a0, b0, c0, nxt, with_t);
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, a1, b1, c1);
+        cur = nxt;
+      }
+    }
+  };
+  // r = z - tau for the 16 keys of block kb (-inf where the row may not look), and dP.
+  auto block_terms = [&](int kt, int kb, const unsigned char* ka, const unsigned char* va, float (&r)[16], f32x16& dp) {
+    f32x16 s = BT::dot_block(ka, kb, qf, lq, lh);
+    dp = BT::dot_block(va, kb, dof, lq, lh);
+    const int jb = kt * kBN + kb * 32 + 4 * lh;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const bool ok = jb + 8 * (i >> 2) + (i & 3) <= lim;
+      r[i] = ok ? fmaf(s[i], p.qscale, -tau) : -INFINITY;
+    }
+  };
+
+  // ---- pass 1: sum p, sum u, sum u dP ----
+  float zsum = 0.f, usum = 0.f, udp = 0.f;
+  tile_loop(false, [&](int kt, const unsigned char* ka, const unsigned char* va, const unsigned char*) {
+    if (p.causal && kt * kBN > wave_row0 + 31) return;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
+      float r[16];
+      f32x16 dp;
+      block_terms(kt, kb, ka, va, r, dp);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float pr, u;
+        bwd_prob<AM>(r[i], p.c0, pr, u);
+        zsum += pr;
+        usum += u;
+        udp = fmaf(u, dp[i], udp);
+      }
+    }
+  });
+  zsum += __shfl_xor(zsum, 32, 64);
+  usum += __shfl_xor(usum, 32, 64);
+  udp += __shfl_xor(udp, 32, 64);
+  const float delta = usum > 0.f ? udp / usum : 0.f;
+  if (live && lh == 0) {
+    p.delta[q_base + qi] = delta;
+    p.zinv[q_base + qi] = zsum > 0.f ? 1.f / zsum : 0.f;
+  }
+
+  // ---- pass 2: dX = u (dP - delta), dQ^T += K^T dX^T ----
+  f32x16 acc[G::kDB];
+#pragma unroll
+  for (int db = 0; db < G::kDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+  tile_loop(true, [&](int kt, const unsigned char* ka, const unsigned char* va, const unsigned char* kta) {
+    if (p.causal && kt * kBN > wave_row0 + 31) return;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
+      float r[16];
+      f32x16 dp;
+      block_terms(kt, kb, ka, va, r, dp);
+      float dx[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float pr, u;
+        bwd_prob<AM>(r[i], p.c0, pr, u);
+        dx[i] = u * (dp[i] - delta);
+      }
+      BT::acc_block(acc, k16 ? kta : ka, kb, dx, lq, lh);
+    }
+  });
+
+  __syncthreads();  // the tile buffers become the transpose scratch: a quarter of a0/b0 per wave pair
+  unsigned char* stage = (wave < 2 ? a0 : b0) + (wave & 1) * (32 * G::kKRow);
+  BT::store_rows(acc, p.sm_scale, stage, dq_rows, wave_row0, N, lane);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dK / dV kernel: grid (blocks of 128 keys, B * Hkv)
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int D, int AM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
+  using BT = BwdTiles<T, D>;
+  using G = TileGeo<T, D>;
+  constexpr bool k16 = G::k16;
+  __shared__ __align__(1024) unsigned char a0[BT::kTile];  // Q tile, row-major
+  __shared__ __align__(1024) unsigned char b0[BT::kTile];  // dO tile, row-major
+  __shared__ __align__(1024) unsigned char c0[k16 ? BT::kTile : 16];  // dO^T (pass 1) or Q^T (pass 2) tile, 16-bit
+  __shared__ __align__(1024) unsigned char a1[BT::kNBuf == 2 ? BT::kTile : 16];
+  __shared__ __align__(1024) unsigned char b1[BT::kNBuf == 2 ? BT::kTile : 16];
+  __shared__ __align__(1024) unsigned char c1[(k16 && BT::kNBuf == 2) ? BT::kTile : 16];
+  __shared__ __align__(16) float scal0[3][kBN];  // tau, 1 / sum p, delta of the tile's queries
+  __shared__ __align__(16) float scal1[3][kBN];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+  const int N = p.N;
+  const int nblk = blockIdx.x;  // early key blocks have the most causal work and come first
+  const int bkv = blockIdx.y;
+  const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
+  const int group = p.Hq / p.Hkv;
+  const int L = bwd_seq_len(p, b);
+  const int n0 = nblk * kBwdRows;
+  const int wave_key0 = n0 + wave * 32;
+  const int kj = wave_key0 + lq;
+  const size_t kv_base = (size_t)bkv * N;
+  unsigned char* dk_rows = reinterpret_cast<unsigned char*>(p.dk) + kv_base * G::kKRow;
+  unsigned char* dv_rows = reinterpret_cast<unsigned char*>(p.dv) + kv_base * G::kKRow;
+
+  if (n0 >= L) {  // padding keys: zero gradient
+    constexpr int kRowDw = D * G::kEB / 4;
+    const int rows = (N - n0) < kBwdRows ? (N - n0) : kBwdRows;
+    uint32_t* k32 = reinterpret_cast<uint32_t*>(dk_rows) + (size_t)n0 * kRowDw;
+    uint32_t* v32 = reinterpret_cast<uint32_t*>(dv_rows) + (size_t)n0 * kRowDw;
+    for (int i = tid; i < rows * kRowDw; i += 256) {
+      k32[i] = 0u;
+      v32[i] = 0u;
+    }
+    return;
+  }
+
+  uint32_t kf[G::kQRegs], vf[G::kQRegs];
+  {
+    const bool ok = kj < N;
+    BT::load_row_frags(p.k, kv_base + (ok ? kj : 0), ok, lh, kf);
+    BT::load_row_frags(p.v, kv_base + (ok ? kj : 0), ok, lh, vf);
+  }
+  const bool key_live = kj < L;
+  const int t_first = p.causal ? n0 / kBN : 0;  // query tiles below the key block see none of its keys
+  const int nt = (L + kBN - 1) / kBN;
+
+  // Runs body(qt, tiles, scalars) over the query tiles [t_first, nt) of query head `hq`.
+  auto tile_loop = [&](int hq, int pass, auto&& body) {
+    const size_t q_base = (size_t)(b * p.Hq + hq) * N;
+    const unsigned char* qg = reinterpret_cast<const unsigned char*>(p.q) + q_base * G::kKRow;
+    const unsigned char* dog = reinterpret_cast<const unsigned char*>(p.dout) + q_base * G::kKRow;
+    const unsigned char* tg =
+        k16 ? reinterpret_cast<const unsigned char*>(pass == 1 ? p.dot : p.qt) + (size_t)(b * p.Hq + hq) * D * p.Npad * 2
+            : nullptr;
+    // column of the forward's tile mask for this key block: is any of its two 64-key tiles kept for the
+    // 128-row block that holds query tile qt?
+    const int32_t* mcol = p.bmask ? p.bmask + (size_t)(b * p.Hq + hq) * p.n_mblk * p.mask_words : nullptr;
+    const int ktile0 = n0 / kBN;
+    auto next_tile = [&](int cur) -> int {
+      int t = cur + 1;
+      if (!mcol) return t < nt ? t : -1;
+      for (; t < nt; ++t) {
+        const uint32_t w = (uint32_t)mcol[(size_t)(t >> 1) * p.mask_words + (ktile0 >> 5)] >> (ktile0 & 31);
+        if (w & 3u) return t;  // (a 128-key block starts on an even tile, so both bits sit in one word)
+      }
+      return -1;
+    };
+    auto issue = [&](unsigned char* a, unsigned char* bb, unsigned char* c, float (*sc)[kBN], int qt) {
+      BT::issue_rows(qg, qt * kBN, N, a, wave, lane);
+      if (pass == 2 || !k16) BT::issue_rows(dog, qt * kBN, N, bb, wave, lane);
+      if constexpr (k16) BT::issue_t(tg + (size_t)qt * BT::kTile, c, wave, lane);
+      if (tid < 3 * kBN) {
+        const int which = tid / kBN, j = tid % kBN;
+        const int qrow = qt * kBN + j;
+        const float* src = which == 0 ? p.taus : (which == 1 ? p.zinv : p.delta);
+        // queries past the sequence end get tau = +inf, which makes every p and u of theirs zero
+        sc[which][j] = qrow < L ? src[q_base + qrow] : (which == 0 ? INFINITY : 0.f);
+      }
+    };
+    __syncthreads();
+    int cur = next_tile(t_first - 1);
+    if (cur >= 0) issue(a0, b0, c0, scal0, cur);
+    while (cur >= 0) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      int nxt = next_tile(cur);
+      if constexpr (BT::kNBuf == 2) {
+        if (nxt >= 0) issue(a1, b1, c1, scal1, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      body(cur, a0, b0, c0, scal0);
+      if constexpr (BT::kNBuf == 1) {
+        __syncthreads();
+        if (nxt >= 0) issue(a0, b0, c0, scal0, nxt);
+        cur = nxt;
+      } else {
+        cur = nxt;
+        if (cur < 0) break;
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        nxt = next_tile(cur);
+        if (nxt >= 0) issue(a0, b0, c0, scal0, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, a1, b1, c1, scal1);
+        cur = nxt;
+      }
+    }
+  };
+  // r = z - tau_i for the 16 queries of block qb against the lane's key (-inf where query i may not see it)
+  auto block_r = [&](int qt, int qb, const unsigned char* qa, const float (*sc)[kBN], float (&r)[16]) {
+    f32x16 s = BT::dot_block(qa, qb, kf, lq, lh);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 tq = *reinterpret_cast<const f32x4*>(&sc[0][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * g + e;
+        const int qrow = qt * kBN + qb * 32 + 8 * g + 4 * lh + e;
+        const bool ok = key_live && (!p.causal || kj <= qrow);
+        r[i] = ok ? fmaf(s[i], p.qscale, -tq[e]) : -INFINITY;
+      }
+    }
+  };
+  auto block_visible = [&](int qt, int qb) {  // does any query of the block see any key of this wave?
+    return !p.causal || qt * kBN + qb * 32 + 31 >= wave_key0;
+  };
+
+  f32x16 acc[G::kDB];
+  unsigned char* stage = (wave < 2 ? a0 : b0) + (wave & 1) * (32 * G::kKRow);
+
+  // ---- pass 1: dV^T += dO^T P ----
+#pragma unroll
+  for (int db = 0; db < G::kDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+  for (int hg = 0; hg < group; ++hg) {
+    tile_loop(kvh * group + hg, 1,
+              [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const float (*sc)[kBN]) {
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) {
+                  if (!block_visible(qt, qb)) continue;
+                  float r[16], w[16];
+                  block_r(qt, qb, qa, sc, r);
+#pragma unroll
+                  for (int g = 0; g < 4; ++g) {
+                    const f32x4 zi = *reinterpret_cast<const f32x4*>(&sc[1][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                      float pr, u;
+                      bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+                      w[4 * g + e] = pr * zi[e];
+                    }
+                  }
+                  BT::acc_block(acc, k16 ? ta : doa, qb, w, lq, lh);
+                }
+              });
+  }
+  __syncthreads();
+  BT::store_rows(acc, 1.f, stage, dv_rows, wave_key0, N, lane);
+
+  // ---- pass 2: dK^T += Q^T dX ----
+#pragma unroll
+  for (int db = 0; db < G::kDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+  for (int hg = 0; hg < group; ++hg) {
+    tile_loop(kvh * group + hg, 2,
+              [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const float (*sc)[kBN]) {
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) {
+                  if (!block_visible(qt, qb)) continue;
+                  float r[16], w[16];
+                  block_r(qt, qb, qa, sc, r);
+                  f32x16 dp = BT::dot_block(doa, qb, vf, lq, lh);
+#pragma unroll
+                  for (int g = 0; g < 4; ++g) {
+                    const f32x4 di = *reinterpret_cast<const f32x4*>(&sc[2][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                      float pr, u;
+                      bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+                      w[4 * g + e] = u * (dp[4 * g + e] - di[e]);
+                    }
+                  }
+                  BT::acc_block(acc, k16 ? ta : qa, qb, w, lq, lh);
+                }
+              });
+  }
+  __syncthreads();
+  BT::store_rows(acc, p.sm_scale, stage, dk_rows, wave_key0, N, lane);
+}
+
+template <typename T, int D> static int launch_attn_bwd_d(const AttnBwdParams& p, int am, hipStream_t s) {
+  const unsigned nq = (unsigned)((p.N + kBwdRows - 1) / kBwdRows);
+  const dim3 gq(nq, (unsigned)(p.B * p.Hq)), gk(nq, (unsigned)(p.B * p.Hkv));
+  if (am == ATT_15) {
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_15>), gq, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_15>), gk, dim3(256), 0, s, p);
+  } else if (am == ATT_2) {
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_2>), gq, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_2>), gk, dim3(256), 0, s, p);
+  } else {
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_GEN>), gq, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_GEN>), gk, dim3(256), 0, s, p);
+  }
+  return 0;
+}
+
+template <typename T> static int launch_attn_bwd(const AttnBwdParams& p, int D, int am, hipStream_t s) {
+  switch (D) {
+    case 16: return launch_attn_bwd_d<T, 16>(p, am, s);
+    case 32: return launch_attn_bwd_d<T, 32>(p, am, s);
+    case 64: return launch_attn_bwd_d<T, 64>(p, am, s);
+    case 128: return launch_attn_bwd_d<T, 128>(p, am, s);
+    case 256: return launch_attn_bwd_d<T, 256>(p, am, s);
+  }
+  return 2;
+}
+
+}  // namespace adsp

@@ -1,0 +1,25 @@
+// Launch parameters of the attention backward kernels.
+#pragma once
+#include <stdint.h>
+
+namespace adsp {
+
+struct AttnBwdParams {
+  const void *q, *k, *v, *dout;
+  const void *kt, *qt, *dot;  // 16-bit path: tile-wise transposed copies of k, q, dout; unused for fp32
+  void *dq, *dk, *dv;
+  const float* taus;  // [B, Hq, N] thresholds of the forward, in z units
+  float* delta;       // [B, Hq, N] written by the dQ kernel, read by the dK/dV kernel
+  float* zinv;        // [B, Hq, N] 1 / sum_j p_ij, likewise
+  const int32_t* bmask;  // [B, Hq, n_mblk, mask_words] tile mask of the forward, or null
+  const void* varlen;
+  int varlen_bits;
+  int B, Hq, Hkv, N, Npad;
+  int n_mblk, mask_words;
+  int causal;
+  float qscale;    // (alpha - 1) / sqrt(D)
+  float sm_scale;  // 1 / sqrt(D)
+  float c0;        // 1 / (alpha - 1)
+};
+
+}  // namespace adsp

@@ -15,6 +15,9 @@
  *                            (adasplash/triton_entmax_v2.py:667-687, kernel :541-617)
  *   adsp_attn_v2_fwd      <- _sparse_attention.forward -> _get_tau, _get_tau_v2, _get_tau_v3,
  *                            _get_output (adasplash/adasplash_v2.py:1243-1438)
+ *   adsp_attn_bwd         <- _sparse_attention.backward -> _bwd_preprocess, _bwd_q_kernel,
+ *                            transpose_bmask, _bwd_kv_kernel (adasplash/adasplash_v2.py:1441-1564) and its
+ *                            generic-alpha twin (adasplash/adasplash_block_mask.py:1079-1210)
  *   adsp_attn_v1_fwd      <- _sparse_attention.forward -> _get_tau,
  *                            compute_bidxs_and_cubcounts, _get_output
  *                            (adasplash/adasplash_block_mask.py:941-1076)
@@ -104,6 +107,29 @@ int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, void* out, flo
                      const void* varlen, int varlen_bits, int B, int H, int N, int D, int dtype, double alpha,
                      int is_causal, int niter, void* workspace, size_t workspace_bytes,
                      unsigned long long* tile_counts, void* stream);
+
+/*
+ * Workspace of adsp_attn_bwd in bytes (tile-wise transposed copies of k, q and dout for the 16-bit
+ * element types; 0 for fp32).
+ */
+size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
+
+/*
+ * Backward of both attention variants: dq, dk, dv for the upstream gradient dout.
+ *   q, dout, dq : [B, Hq, N, D]; k, v, dk, dv : [B, Hkv, N, D] (Hq == Hkv for the block-mask variant).
+ *   taus, bmask : what the forward wrote for the same inputs (bmask may be NULL: every tile is visited).
+ *   delta, zinv : [B, Hq, N] fp32 scratch owned by the caller; receive sum_j u_ij dP_ij / sum_j u_ij and
+ *                 1 / sum_j p_ij per query row.
+ *   alpha, is_causal : 1.5 / 1 for the AdaSplash-2 path, any alpha in (1, 2] for the block-mask path.
+ * Rows of dout past a sequence's valid length must be finite (they are multiplied by zero); gradient rows
+ * past the valid length are written as zeros.  Replaces the four launches at
+ * adasplash/adasplash_v2.py:1456-1562 (delta from out2, dq, mask transpose, dk/dv with the GQA group loop)
+ * and adasplash/adasplash_block_mask.py:1079-1210.
+ */
+int adsp_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* taus,
+                  const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
+                  float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
+                  int is_causal, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

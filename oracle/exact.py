@@ -167,6 +167,39 @@ def dense_entmax_attention(q, k, v, alpha=1.5, is_causal=False, varlen=None, dty
     return out
 
 
+def dense_entmax_attention_grads(q, k, v, dout, alpha=1.5, is_causal=False, varlen=None, dtype=torch.float64):
+    """Gradients (dq, dk, dv) of ``dense_entmax_attention`` for the upstream gradient ``dout``.
+
+    Closed form of the entmax Jacobian: with u = p^(2 - alpha), dX = u * (dP - sum(u dP) / sum(u)) on the
+    scaled scores x = q.k / sqrt(D), where dP = dout . v^T (what adasplash/adasplash_v2.py:1062-1068 and
+    :1196-1215 compute with u = [z - tau]_+ for alpha = 1.5).  Checked in tests/test_oracle.py against central
+    finite differences of the forward oracle.  Padded query rows contribute nothing; padded keys get zero.
+    """
+    out, probs, tau, scores = dense_entmax_attention(q, k, v, alpha, is_causal, varlen, dtype, return_aux=True)
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    g = Hq // Hkv
+    qd, kd, vd, dod = (t.to(dtype) for t in (q, k, v, dout))
+    ke = kd.repeat_interleave(g, dim=1) if g > 1 else kd
+    ve = vd.repeat_interleave(g, dim=1) if g > 1 else vd
+    if varlen is not None:
+        row_valid = (torch.arange(N)[None, :] < varlen.to(torch.long)[:, None])[:, None, :, None]
+        dod = dod.masked_fill(~row_valid, 0.0)
+        probs = probs.masked_fill(~row_valid, 0.0)
+    u = torch.where(probs > 0, probs.clamp_min(1e-300) ** (2.0 - alpha), torch.zeros_like(probs))
+    dp = torch.matmul(dod, ve.transpose(-1, -2))
+    delta = (u * dp).sum(-1, keepdim=True) / u.sum(-1, keepdim=True).clamp_min(1e-300)
+    dx = u * (dp - delta)
+    sm = 1.0 / math.sqrt(D)
+    dq = torch.matmul(dx, ke) * sm
+    dk = torch.matmul(dx.transpose(-1, -2), qd) * sm
+    dv = torch.matmul(probs.transpose(-1, -2), dod)
+    if g > 1:
+        dk = dk.view(B, Hkv, g, N, D).sum(2)
+        dv = dv.view(B, Hkv, g, N, D).sum(2)
+    return dq, dk, dv
+
+
 def dense_entmax_attention_loop(q, k, v, alpha=1.5, is_causal=False, varlen=None):
     """Brute-force per-row restatement (python loops, tiny sizes only) used to pin the dense version."""
     B, Hq, N, D = q.shape

@@ -1,0 +1,107 @@
+"""GPU parity of the attention backward (dq, dk, dv) against the oracle's closed-form entmax gradients,
+which tests/test_oracle.py pins by finite differences of the forward oracle.
+
+Tolerances on max |got - oracle|: fp32 1e-4 (what the reference asks of its own kernels against
+entmax_bisect's autograd, tests/test_adasplash_v2.py:146-179; it has no 16-bit gradient test), 16-bit types
+4e-2 on the magnitude-aware scale of tests/gpu_util.max_err: P and dX are rounded to the element type before
+their MFMA, as the reference does (adasplash/adasplash_v2.py:1066-1068), and the sums run over hundreds of
+such terms with |g| up to ~10."""
+
+import pytest
+import torch
+
+import adasplash_amd as A
+from oracle import exact
+from tests.gpu_util import DEV, max_err
+
+pytestmark = pytest.mark.gpu
+
+
+def grad_tol(dtype):
+    return 1e-4 if dtype == torch.float32 else 4e-2
+
+
+def run_case(alpha, causal, B, Hq, Hkv, N, D, dtype, varlen=None, version=1, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (scale * torch.randn(B, Hq, N, D, generator=g)).to(dtype)
+    k = (scale * torch.randn(B, Hkv, N, D, generator=g)).to(dtype)
+    v = torch.randn(B, Hkv, N, D, generator=g).to(dtype)
+    do = torch.randn(B, Hq, N, D, generator=g).to(dtype)
+    qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    vl = varlen.to(DEV) if varlen is not None else None
+    if version == 2:
+        out = A.adasplash_v2(qg, kg, vg, niter=10, varlen=vl)
+    else:
+        out = A.adasplash_v1(qg, kg, vg, alpha=alpha, is_causal=causal, varlen=vl, niter=20)
+    out.backward(do.to(DEV))
+    want = exact.dense_entmax_attention_grads(q, k, v, do, alpha, causal, varlen)
+    return (qg.grad, kg.grad, vg.grad), want
+
+
+def check(got, want, dtype):
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert g.dtype == dtype and g.shape == w.shape
+        assert torch.isfinite(g).all(), name
+        assert max_err(g, w) < grad_tol(dtype), name
+
+
+@pytest.mark.parametrize("N,D", [(128, 64), (256, 128), (512, 32), (128, 16), (128, 256)])
+def test_v2_backward_fp32(N, D):
+    got, want = run_case(1.5, True, 1, 2, 2, N, D, torch.float32, version=2)
+    check(got, want, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,D", [(256, 64), (512, 128), (256, 256)])
+def test_v2_backward_16bit(dtype, N, D):
+    got, want = run_case(1.5, True, 1, 2, 2, N, D, dtype, version=2)
+    check(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_v2_backward_gqa_and_varlen(dtype):
+    # adasplash/adasplash_v2.py:1180-1188: dk / dv accumulate over the query heads of a K/V head;
+    # lengths that end inside a 128-row block, inside a 64-key tile, and a full one
+    varlen = torch.tensor([300, 77, 384], dtype=torch.int32)
+    got, want = run_case(1.5, True, 3, 8, 2, 384, 64, dtype, varlen=varlen, version=2)
+    check(got, want, dtype)
+    for b, L in enumerate(varlen.tolist()):
+        for g in got:
+            assert (g[b, :, L:] == 0).all()  # padded rows get exactly zero gradient
+
+
+def test_v2_backward_matches_reference_test_shape():
+    # tests/test_adasplash_v2.py:146-179 at its smallest length
+    got, want = run_case(1.5, True, 2, 2, 2, 1024, 64, torch.float32, version=2, seed=42)
+    check(got, want, torch.float32)
+
+
+@pytest.mark.parametrize("alpha", [1.333, 1.5, 2.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_v1_backward_alphas(alpha, causal):
+    got, want = run_case(alpha, causal, 1, 2, 2, 256, 64, torch.float32)
+    check(got, want, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_v1_backward_varlen_and_sparse_rows(dtype):
+    # a higher temperature makes most tiles drop out of the forward's mask, which the backward reuses
+    varlen = torch.tensor([512, 200], dtype=torch.int64)
+    got, want = run_case(1.333, False, 2, 2, 2, 512, 64, dtype, varlen=varlen, scale=2.0)
+    check(got, want, dtype)
+
+
+def test_zero_upstream_gradient_gives_zero():
+    q, k, v = (torch.randn(1, 2, 128, 64, device=DEV, requires_grad=True) for _ in range(3))
+    out = A.adasplash(q, k, v)
+    out.backward(torch.zeros_like(out))
+    assert all((t.grad == 0).all() for t in (q, k, v))
+
+
+def test_gradient_of_the_sum_vanishes_for_q_and_k():
+    # rows of P sum to one, so with v = const the output does not depend on q and k
+    q, k = (torch.randn(1, 2, 256, 64, device=DEV, requires_grad=True) for _ in range(2))
+    v = torch.ones(1, 2, 256, 64, device=DEV, requires_grad=True)
+    out = A.adasplash_v1(q, k, v, alpha=1.5, is_causal=True, niter=20)
+    out.backward(torch.randn(1, 2, 256, 64, device=DEV))
+    assert q.grad.abs().max() < 1e-4 and k.grad.abs().max() < 1e-4

@@ -174,3 +174,40 @@ def test_oracle_reproduces_the_committed_golden_vectors(golden_dir):
     g = np.load(golden_dir / "attn_v2_b1h8n128d64.npz")
     out = exact.dense_entmax_attention(*(torch.tensor(g[n]) for n in "qkv"), 1.5, True)
     assert np.abs(out.float().numpy() - g["out"]).max() < 1e-6
+
+
+@pytest.mark.parametrize(
+    "alpha,causal,shape,varlen",
+    [
+        (1.5, True, (1, 2, 1, 12, 4), None),
+        (2.0, False, (1, 1, 1, 10, 4), None),
+        (1.333, True, (2, 2, 2, 9, 4), [9, 6]),
+    ],
+)
+def test_closed_form_gradients_match_finite_differences(alpha, causal, shape, varlen):
+    # pins dense_entmax_attention_grads (a dropped -delta term, a missing 1/sqrt(D), a transposed dk or a
+    # wrong GQA reduction all fail here): central differences of the forward oracle in fp64
+    B, Hq, Hkv, N, D = shape
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, Hq, N, D, generator=g, dtype=torch.float64)
+    k = torch.randn(B, Hkv, N, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, Hkv, N, D, generator=g, dtype=torch.float64)
+    do = torch.randn(B, Hq, N, D, generator=g, dtype=torch.float64)
+    vl = torch.tensor(varlen) if varlen is not None else None
+    grads = exact.dense_entmax_attention_grads(q, k, v, do, alpha, causal, vl)
+
+    def loss():
+        return (exact.dense_entmax_attention(q, k, v, alpha, causal, vl) * do).sum().item()
+
+    eps = 1e-6
+    for t, gr in zip((q, k, v), grads):
+        flat, num = t.view(-1), torch.zeros(t.numel(), dtype=torch.float64)
+        for i in range(flat.numel()):
+            old = flat[i].item()
+            flat[i] = old + eps
+            fp = loss()
+            flat[i] = old - eps
+            fm = loss()
+            flat[i] = old
+            num[i] = (fp - fm) / (2 * eps)
+        assert (num.view_as(gr) - gr).abs().max() < 1e-7
