@@ -130,7 +130,13 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(Att
   if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return;
   const int hg = (int)(logical % group);
   const int mi = (int)((logical / group) % n_mblk);
-  const int bkv = (int)(logical / ((long long)group * n_mblk));
+  // K/V heads are dealt to the XCDs round-robin rather than in contiguous runs: with right-padded
+  // batches a contiguous run is one batch item, and the XCD that drew the longest sequence would finish last
+  int bkv = (int)(logical / ((long long)group * n_mblk));
+  {
+    const int units = p.B * p.Hkv;
+    if (units % 8 == 0) bkv = (bkv % (units / 8)) * 8 + bkv / (units / 8);
+  }
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int h = kvh * group + hg;
   const int mblk = n_mblk - 1 - mi;
