@@ -1,8 +1,8 @@
 // Fused sparse entmax attention forward for gfx950 (one kernel: threshold solver + output).
 //
 // Work decomposition
-//   workgroup = NW waves (8, or 4 for the register-heavy shapes), owns 32*NW consecutive query rows of
-//   one (batch, head); wave w owns rows [32w, 32w+32); inside a wave, lane l holds query row (l & 31)
+//   workgroup = 4 waves, owns 128 consecutive query rows of one (batch, head) and is sized so that two
+//   workgroups fit a CU; wave w owns rows [32w, 32w+32); inside a wave, lane l holds query row (l & 31)
 //   and, of every 32-key block, the 16 keys {8g + 4(l >> 5) + r : g, r in 0..3} -- the C layout of the
 //   32x32 MFMA when the product is taken as S^T = K Q^T.  All per-row quantities (max, histogram,
 //   Halley sums, tau, sum of p) are therefore lane-local accumulators that need one cross-lane add
@@ -75,10 +75,13 @@ template <typename T, int D> struct TileGeo {
   static constexpr int kVRows = k16 ? D : kBN;
   static constexpr int kVTile = kVRows * kVRow;
   static constexpr int kNBuf = (2 * (kKTile + kVTile) <= 144 * 1024) ? 2 : 1;
-  // eight waves (two per SIMD, <= 256 registers each) unless the shape needs the full register file
-  static constexpr int kNW = (kNBuf == 1 || (!k16 && D >= 128) || (k16 && D >= 256)) ? 4 : 8;
+  // Four waves of at most 256 registers: two workgroups share a CU (LDS permitting), one wave of each per
+  // SIMD.  Their barriers are independent, so one workgroup's wait for a tile overlaps the other's MFMAs.
+  static constexpr int kNW = 4;
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
+  // shapes whose live state fits 256 registers are held to two waves per SIMD; the others take what they need
+  static constexpr int kMinWaves = ((k16 && D <= 128) || (!k16 && D <= 64)) ? 2 : 1;
   static constexpr int kQRegs = k16 ? (D / 16) * 4 : D / 2;  // dwords of Q held per lane
   static constexpr int kDB = D >= 32 ? D / 32 : 1;           // 32-wide d blocks of the output
   static constexpr int kKLoads = kKTile / 1024;              // wave-level 1 KB DMA instructions per K tile
@@ -97,7 +100,7 @@ template <int AM> __device__ __forceinline__ float attn_prob(float r, float qs, 
 }
 
 template <typename T, int D, int AM>
-__global__ __launch_bounds__((TileGeo<T, D>::kThreads)) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_waves_per_eu(TileGeo<T, D>::kMinWaves, 2))) void attn_fwd_kernel(AttnParams p) {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
   using VS = Swz<G::kVRow>;
