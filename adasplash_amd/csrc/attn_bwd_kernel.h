@@ -49,7 +49,10 @@ template <typename T, int D> struct BwdTiles {
   static constexpr int kTile = G::kKTile;  // bytes of a [64][D] tile, in either orientation
   static constexpr int kNW = kBwdRows / 32;
   static constexpr int kSlots = k16 ? 3 : 2;  // tiles per pipeline stage
-  static constexpr int kNBuf = (2 * kSlots * kTile <= 144 * 1024) ? 2 : 1;
+  // Double-buffer only while two workgroups still fit a CU: a second resident workgroup hides a tile's
+  // load latency better than a second stage does, and brings a second wave to every SIMD.
+  static constexpr int kNBuf = (2 * kSlots * kTile <= 64 * 1024) ? 2 : 1;
+  static constexpr int kMinWaves = G::kMinWaves;
   static constexpr int kLoads = kTile / 1024;
 
   // DMA of rows [row0, row0 + 64) of a row-major [N][D] tensor into a swizzled tile.
@@ -212,7 +215,7 @@ __device__ __forceinline__ int bwd_seq_len(const AttnBwdParams& p, int b) {
 // dQ kernel: grid (row blocks of 128 queries, B * Hq)
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, int D, int AM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void attn_bwd_dq_kernel(AttnBwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T, D>::kMinWaves), 2))) void attn_bwd_dq_kernel(AttnBwdParams p) {
   using BT = BwdTiles<T, D>;
   using G = TileGeo<T, D>;
   constexpr bool k16 = G::k16;
@@ -391,7 +394,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
 // dK / dV kernel: grid (blocks of 128 keys, B * Hkv)
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, int D, int AM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T, D>::kMinWaves), 2))) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
   using BT = BwdTiles<T, D>;
   using G = TileGeo<T, D>;
   constexpr bool k16 = G::k16;
