@@ -10,7 +10,8 @@ Workloads (``--workload``):
   c3   adasplash_v2 causal MHA, B=4 H=16 N=4096 D=64 bf16, q pre-scaled by 1/sqrt(D)
   c5   adasplash_v1 non-causal alpha=1.333 niter=10, B=2 H=16 N=16384 D=64 bf16, q,k x3
   c2   entmax rows x[16384, 8192] = 4*N(0,1), bf16 and fp32, alpha in {1.5, 2}
-The default run also times the entmax rows workload (c2) and reports it under ``extra``.
+  c4_bwd, c3_bwd   dq, dk, dv of the c4 / c3 forward (2.5 x its dense-equivalent FLOPs per step)
+The default run also times the entmax rows workload (c2) and the c4 backward and reports them under ``extra``.
 
 Dense-equivalent FLOPs of causal attention = 2 * Hq * D * sum_b L_b^2 (QK^T and PV, each halved by
 causality); non-causal = 4 * B * H * N^2 * D.  Rows bytes = rows * cols * (sizeof(in) + sizeof(out)).
@@ -87,7 +88,7 @@ def make_c5(device, seed=42):
     return (q, k, v), flops, cfg
 
 
-def bench_attention(name, steps, warmup, device):
+def bench_attention(name, steps, warmup, device, backward=False):
     import adasplash_amd as A
 
     if name == "c4":
@@ -99,6 +100,19 @@ def bench_attention(name, steps, warmup, device):
     else:
         (q, k, v), flops, cfg = make_c5(device)
         fn = lambda: A.adasplash_v1(q, k, v, alpha=1.333, is_causal=False, niter=10)  # noqa: E731
+    if backward:
+        # one step = dq, dk, dv for a fixed upstream gradient (the forward runs once, outside the timed region);
+        # dense-equivalent work: S recomputed, dP, dV, dK, dQ = 2.5 x the forward's two products
+        from adasplash_amd import _attention
+
+        assert name in ("c4", "c3")
+        out, taus, bmask = _attention.launch_forward(q, k, v, version=2, alpha=1.5, is_causal=True, niter=1,
+                                                     varlen=varlen)
+        dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(7)).to(q.dtype).to(device)
+        fn = lambda: _attention.launch_backward(q, k, v, dout, taus, bmask, alpha=1.5, is_causal=True,  # noqa: E731
+                                                varlen=varlen)
+        flops = 2.5 * flops
+        cfg = dict(cfg, workload=cfg["workload"].replace("fwd", "bwd (dq, dk, dv)"))
     ms, wall_ms = _events_ms(fn, steps, warmup)
     tflops = flops / (ms * 1e-3) / 1e12
     res = {"ms_per_step": ms, "wall_ms_per_step": wall_ms, "eff_tflops": tflops, "flops_per_step": flops,
@@ -173,7 +187,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd"])
     ap.add_argument("--no-extra", action="store_true", help="skip the entmax-rows and CPU-baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -208,18 +222,26 @@ def main():
                                   "kernel": "entmax_rows_reg_kernel", "bytes_per_launch": best["bytes"]},
                      "extra": {"entmax_rows": rows}})
     else:
-        res = bench_attention(args.workload, args.steps, args.warmup, device)
+        bwd = args.workload.endswith("_bwd")
+        res = bench_attention(args.workload[:2], args.steps, args.warmup, device, backward=bwd)
         line.update({"value": res["eff_tflops"], "unit": "TFLOP/s", "ms_per_step": res["ms_per_step"],
                      "dtype": "bf16", "config": res["config"],
                      "roofline": {"bound": "mfma", "achieved": res["eff_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                                   "unit": "TFLOP/s", "frac": res["frac_mfma_peak"],
                                   "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
-                                  "kernel": "attn_fwd_kernel", "flops_per_launch": res["flops_per_step"]},
+                                  "kernel": "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel" if bwd else "attn_fwd_kernel",
+                                  "flops_per_launch": res["flops_per_step"]},
                      "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k == "wall_ms_per_step"}})
         if not args.no_extra:
             del res
             torch.cuda.empty_cache()
             line["extra"]["entmax_rows"] = bench_rows(args.steps, args.warmup, device)
+            if args.workload == "c4":
+                b = bench_attention("c4", max(3, args.steps // 2), 1, device, backward=True)
+                line["extra"]["attention_backward"] = {k: b[k] for k in ("ms_per_step", "eff_tflops", "frac_mfma_peak",
+                                                                         "flops_per_step")}
+                del b
+                torch.cuda.empty_cache()
     if not args.no_extra:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
