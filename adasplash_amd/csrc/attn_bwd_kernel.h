@@ -211,8 +211,24 @@ __device__ __forceinline__ int bwd_seq_len(const AttnBwdParams& p, int b) {
   return L;
 }
 
+
+// Hardware block ids are dealt round-robin to the 8 XCDs (each with its own L2).  Blocks are renumbered so
+// that every XCD works through whole K/V heads, one after the other, and the K/V heads themselves are dealt
+// round-robin to the XCDs, which keeps right-padded batches balanced.  Returns false for the padding blocks
+// of the grid; `inner` = blocks per K/V head, `unit` / `in_unit` = K/V head index and block index inside it.
+__device__ __forceinline__ bool bwd_block_map(int units, int inner, int& unit, int& in_unit) {
+  const long long total = (long long)units * inner;
+  const long long per_xcd = (total + 7) / 8;
+  const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return false;
+  unit = (int)(logical / inner);
+  in_unit = (int)(logical % inner);
+  if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
+  return true;
+}
+
 // ---------------------------------------------------------------------------------------------------------
-// dQ kernel: grid (row blocks of 128 queries, B * Hq)
+// dQ kernel: one block per (K/V head, query head in its group, row block of 128 queries)
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, int D, int AM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T, D>::kMinWaves), 2))) void attn_bwd_dq_kernel(AttnBwdParams p) {
@@ -231,10 +247,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
   const int N = p.N;
   const int n_blk = (N + kBwdRows - 1) / kBwdRows;
-  const int mblk = n_blk - 1 - (int)blockIdx.x;  // the longest causal rows first
-  const int bh = blockIdx.y;
-  const int b = bh / p.Hq, h = bh % p.Hq;
-  const int kvh = h / (p.Hq / p.Hkv);
+  const int group = p.Hq / p.Hkv;
+  int bkv, in_unit;
+  if (!bwd_block_map(p.B * p.Hkv, n_blk * group, bkv, in_unit)) return;
+  const int mblk = n_blk - 1 - in_unit / group;  // the longest causal rows first; a group's heads side by side
+  const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
+  const int h = kvh * group + in_unit % group;
+  const int bh = b * p.Hq + h;
   const int L = bwd_seq_len(p, b);
   const int m0 = mblk * kBwdRows;
   const int wave_row0 = m0 + wave * 32;
@@ -391,7 +410,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// dK / dV kernel: grid (blocks of 128 keys, B * Hkv)
+// dK / dV kernel: one block per (K/V head, block of 128 keys)
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, int D, int AM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T, D>::kMinWaves), 2))) void attn_bwd_dkdv_kernel(AttnBwdParams p) {
@@ -411,8 +430,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
   const int N = p.N;
-  const int nblk = blockIdx.x;  // early key blocks have the most causal work and come first
-  const int bkv = blockIdx.y;
+  int bkv, nblk;  // early key blocks have the most causal work and come first
+  if (!bwd_block_map(p.B * p.Hkv, (N + kBwdRows - 1) / kBwdRows, bkv, nblk)) return;
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int group = p.Hq / p.Hkv;
   const int L = bwd_seq_len(p, b);
@@ -592,8 +611,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
 }
 
 template <typename T, int D> static int launch_attn_bwd_d(const AttnBwdParams& p, int am, hipStream_t s) {
-  const unsigned nq = (unsigned)((p.N + kBwdRows - 1) / kBwdRows);
-  const dim3 gq(nq, (unsigned)(p.B * p.Hq)), gk(nq, (unsigned)(p.B * p.Hkv));
+  const long long nq = (p.N + kBwdRows - 1) / kBwdRows;
+  const dim3 gq((unsigned)(((long long)p.B * p.Hq * nq + 7) / 8 * 8)), gk((unsigned)(((long long)p.B * p.Hkv * nq + 7) / 8 * 8));
   if (am == ATT_15) {
     hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_15>), gq, dim3(256), 0, s, p);
     hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_15>), gk, dim3(256), 0, s, p);
