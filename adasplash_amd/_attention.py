@@ -65,7 +65,7 @@ def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
     dout = dout.to(q.dtype).contiguous()
     if varlen is not None:
         valid = torch.arange(N, device=q.device)[None, :] < varlen.to(torch.long)[:, None]
-        dout = dout * valid[:, None, :, None].to(dout.dtype)
+        dout = torch.where(valid[:, None, :, None], dout, torch.zeros((), device=q.device, dtype=dout.dtype))
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)

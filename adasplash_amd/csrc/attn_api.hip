@@ -16,21 +16,29 @@ int launch_attn_bwd_f32(const AttnBwdParams& p, int D, int am, hipStream_t s);
 // Tile-wise key-major, MFMA-ordered copy of V for the 16-bit path.  Keys are cut in tiles of 64; a tile
 // is stored as one contiguous [D][64] block (so the kernel fetches it with contiguous kilobyte copies):
 //   vt[bh, kt, d, pos(n % 64)] = v[bh, n, d],  kt = n / 64,
-//   pos(16s + 8a + 4h + r) = 16s + 8h + 4a + r,  zero for n >= N.
+//   pos(16s + 8a + 4h + r) = 16s + 8h + 4a + r,  zero for n >= the sequence's valid length (so that
+//   whatever the caller left in the padding rows never meets an MFMA).
 // With this order a lane of the PV product reads its 8 keys {16s + 4h + r, 16s + 8 + 4h + r} of one
 // d row as one 16-byte LDS access.
 __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
-                                                        int N, int Npad, int D) {
+                                                        int N, int Npad, int D, const void* varlen, int varlen_bits,
+                                                        int heads) {
   extern __shared__ __align__(16) unsigned char smem[];
   uint16_t* tile = reinterpret_cast<uint16_t*>(smem);  // [64][D + 2]
   const int pitch = D + 2;
   const int kt = blockIdx.x;
   const size_t bh = blockIdx.y;
   const uint16_t* vsrc = v + bh * (size_t)N * D;
+  int L = N;
+  if (varlen) {
+    const size_t b = bh / heads;
+    long long l = varlen_bits == 64 ? ((const long long*)varlen)[b] : (long long)((const int*)varlen)[b];
+    L = (int)(l < 0 ? 0 : (l > N ? N : l));
+  }
   for (int i = threadIdx.x; i < 64 * D; i += 256) {
     int key = i / D, d = i % D;
     int gk = kt * 64 + key;
-    tile[key * pitch + d] = gk < N ? vsrc[(size_t)gk * D + d] : (uint16_t)0;
+    tile[key * pitch + d] = gk < L ? vsrc[(size_t)gk * D + d] : (uint16_t)0;
   }
   __syncthreads();
   uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64 * D;
@@ -90,7 +98,7 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
     p.vt = workspace;
     hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hkv)), dim3(256),
-                       (size_t)64 * (D + 2) * 2, s, (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D);
+                       (size_t)64 * (D + 2) * 2, s, (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv);
   }
   int rc = dtype == ADSP_BF16 ? launch_attn_bf16(p, D, am, s)
                               : (dtype == ADSP_F16 ? launch_attn_f16(p, D, am, s) : launch_attn_f32(p, D, am, s));
@@ -183,11 +191,11 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
     const size_t shm = (size_t)64 * (D + 2) * 2;
     hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hkv)), dim3(256), shm, s,
-                       (const uint16_t*)k, kt, N, p.Npad, D);
+                       (const uint16_t*)k, kt, N, p.Npad, D, varlen, varlen_bits, Hkv);
     hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hq)), dim3(256), shm, s,
-                       (const uint16_t*)q, qt, N, p.Npad, D);
+                       (const uint16_t*)q, qt, N, p.Npad, D, varlen, varlen_bits, Hq);
     hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hq)), dim3(256), shm, s,
-                       (const uint16_t*)dout, dot, N, p.Npad, D);
+                       (const uint16_t*)dout, dot, N, p.Npad, D, varlen, varlen_bits, Hq);
     p.kt = kt;
     p.qt = qt;
     p.dot = dot;

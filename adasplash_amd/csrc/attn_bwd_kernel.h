@@ -134,9 +134,10 @@ template <typename T, int D> struct BwdTiles {
   }
   // o^T[d][lane row] += sum over the 32 tile rows of block kb of  tile[row][d] * w[row][lane row], where
   // w holds the lane's 16 values in the accumulator order of dot_block.  16-bit: `tile` is the transposed
-  // tile; fp32: the row-major one.
+  // tile (its padding rows are zero); fp32: the row-major one, of which only the first `rows_valid` rows
+  // are used (padding rows of the caller's tensors may hold anything).
   static __device__ __forceinline__ void acc_block(f32x16 (&o)[G::kDB], const unsigned char* tile, int kb,
-                                                   const float (&w)[16], int lq, int lh) {
+                                                   const float (&w)[16], int lq, int lh, int rows_valid) {
     if constexpr (k16) {
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
@@ -159,6 +160,7 @@ template <typename T, int D> struct BwdTiles {
           const int dcol = db * 32 + lq;
           float a = 0.f;
           if (D >= 32 || dcol < D) a = *reinterpret_cast<const float*>(tile + KS::off(row, dcol >> 2) + (dcol & 3) * 4);
+          if (row >= rows_valid) a = 0.f;
           o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, w[i], o[db], 0, 0, 0);
         }
       }
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
 
   uint32_t qf[G::kQRegs], dof[G::kQRegs];
   {
-    const bool ok = qi < N;
+    const bool ok = qi < L;  // padding rows take no part
     BT::load_row_frags(p.q, q_base + (ok ? qi : 0), ok, lh, qf);
     BT::load_row_frags(p.dout, q_base + (ok ? qi : 0), ok, lh, dof);
   }
@@ -347,6 +349,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     for (int i = 0; i < 16; ++i) {
       const bool ok = jb + 8 * (i >> 2) + (i & 3) <= lim;
       r[i] = ok ? fmaf(s[i], p.qscale, -tau) : -INFINITY;
+      dp[i] = ok ? dp[i] : 0.f;  // keys past the end may hold anything
     }
   };
 
@@ -400,7 +403,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
         bwd_prob<AM>(r[i], p.c0, pr, u);
         dx[i] = u * (dp[i] - delta);
       }
-      BT::acc_block(acc, k16 ? kta : ka, kb, dx, lq, lh);
+      BT::acc_block(acc, k16 ? kta : ka, kb, dx, lq, lh, L - kt * kBN);
     }
   });
 
@@ -456,7 +459,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
 
   uint32_t kf[G::kQRegs], vf[G::kQRegs];
   {
-    const bool ok = kj < N;
+    const bool ok = kj < L;  // padding keys take no part
     BT::load_row_frags(p.k, kv_base + (ok ? kj : 0), ok, lh, kf);
     BT::load_row_frags(p.v, kv_base + (ok ? kj : 0), ok, lh, vf);
   }
@@ -536,7 +539,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
       for (int e = 0; e < 4; ++e) {
         const int i = 4 * g + e;
         const int qrow = qt * kBN + qb * 32 + 8 * g + 4 * lh + e;
-        const bool ok = key_live && (!p.causal || kj <= qrow);
+        const bool ok = key_live && qrow < L && (!p.causal || kj <= qrow);
         r[i] = ok ? fmaf(s[i], p.qscale, -tq[e]) : -INFINITY;
       }
     }
@@ -571,7 +574,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
                       w[4 * g + e] = pr * zi[e];
                     }
                   }
-                  BT::acc_block(acc, k16 ? ta : doa, qb, w, lq, lh);
+                  BT::acc_block(acc, k16 ? ta : doa, qb, w, lq, lh, L - qt * kBN);
                 }
               });
   }
@@ -599,10 +602,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
                     for (int e = 0; e < 4; ++e) {
                       float pr, u;
                       bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
-                      w[4 * g + e] = u * (dp[4 * g + e] - di[e]);
+                      w[4 * g + e] = u > 0.f ? u * (dp[4 * g + e] - di[e]) : 0.f;
                     }
                   }
-                  BT::acc_block(acc, k16 ? ta : qa, qb, w, lq, lh);
+                  BT::acc_block(acc, k16 ? ta : qa, qb, w, lq, lh, L - qt * kBN);
                 }
               });
   }

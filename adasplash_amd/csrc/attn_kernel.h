@@ -624,6 +624,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
               float a = 0.f;
               if (D >= 32 || dcol < D)
                 a = *reinterpret_cast<const float*>(vt_lds + VS::off(key, dcol >> 2) + (dcol & 3) * 4);
+              if (kt * kBN + key >= L) a = 0.f;  // padding rows of v may hold anything
               o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, pv[i], o[db], 0, 0, 0);
             }
           }

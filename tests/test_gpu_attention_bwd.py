@@ -105,3 +105,31 @@ def test_gradient_of_the_sum_vanishes_for_q_and_k():
     out = A.adasplash_v1(q, k, v, alpha=1.5, is_causal=True, niter=20)
     out.backward(torch.randn(1, 2, 256, 64, device=DEV))
     assert q.grad.abs().max() < 1e-4 and k.grad.abs().max() < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("version", [1, 2])
+def test_padding_rows_may_hold_anything(dtype, version):
+    # the reference never reads past a sequence's valid length (masked loads, adasplash/adasplash_v2.py:
+    # 1030-1033, 1194-1207): NaNs parked in the padding of q, k, v and of the upstream gradient must not leak
+    g = torch.Generator().manual_seed(5)
+    B, H, N, D = 2, 2, 256, 64
+    varlen = torch.tensor([150, 256], dtype=torch.int32)
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dtype) for _ in range(4))
+    dirty = [t.clone() for t in (q, k, v, do)]
+    for t in dirty:
+        t[0, :, 150:] = float("nan")
+
+    def run(ts):
+        qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in ts[:3])
+        if version == 2:
+            out = A.adasplash_v2(qg, kg, vg, niter=10, varlen=varlen.to(DEV))
+        else:
+            out = A.adasplash_v1(qg, kg, vg, alpha=1.5, is_causal=False, varlen=varlen.to(DEV), niter=20)
+        out.backward(ts[3].to(DEV))
+        return out.detach(), qg.grad, kg.grad, vg.grad
+
+    clean, soiled = run((q, k, v, do)), run(dirty)
+    for a, b in zip(clean, soiled):
+        assert torch.isfinite(b).all()
+        assert torch.equal(a, b)
