@@ -500,7 +500,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     for (int it = 0; it < p.niter; ++it) {
       const float init = -br.t * inv_qs;
       const float dl = (br.lo - br.t) * inv_qs;  // z > lo  <=>  (s - t_raw) > dl
-      const bool refine = it == p.niter - 1 || mask_cur == nullptr;
+      const bool refine = true;  // every step tightens the tile mask to {z > lower bound} for the next pass
       float a0 = 0.f, a1 = 0.f, a2 = 0.f;
       int cnt_pos = 0;
       tile_loop(mask_cur, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
