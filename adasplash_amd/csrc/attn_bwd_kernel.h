@@ -480,9 +480,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     const int32_t* mcol = p.bmask ? p.bmask + (size_t)(b * p.Hq + hq) * p.n_mblk * p.mask_words : nullptr;
     const int ktile0 = n0 / kBN;
     auto next_tile = [&](int cur) -> int {
-      int t = cur + 1;
-      if (!mcol) return t < nt ? t : -1;
-      for (; t < nt; ++t) {
+      // Query tiles are walked from the last one down: every key block of a K/V head then starts on the
+      // same tile and the workgroups that run side by side on an XCD read the same Q / dO tiles at about
+      // the same time, out of its L2 (walking upwards, each would start at its own diagonal).
+      int t = cur - 1;
+      if (!mcol) return t >= t_first ? t : -1;
+      for (; t >= t_first; --t) {
         const uint32_t w = (uint32_t)mcol[(size_t)(t >> 1) * p.mask_words + (ktile0 >> 5)] >> (ktile0 & 31);
         if (w & 3u) return t;  // (a 128-key block starts on an even tile, so both bits sit in one word)
       }
@@ -492,16 +495,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
       BT::issue_rows(qg, qt * kBN, N, a, wave, lane);
       if (pass == 2 || !k16) BT::issue_rows(dog, qt * kBN, N, bb, wave, lane);
       if constexpr (k16) BT::issue_t(tg + (size_t)qt * BT::kTile, c, wave, lane);
-      if (tid < 3 * kBN) {
-        const int which = tid / kBN, j = tid % kBN;
-        const int qrow = qt * kBN + j;
-        const float* src = which == 0 ? p.taus : (which == 1 ? p.zinv : p.delta);
-        // queries past the sequence end get tau = +inf, which makes every p and u of theirs zero
-        sc[which][j] = qrow < L ? src[q_base + qrow] : (which == 0 ? INFINITY : 0.f);
+      // tau, 1 / sum p and delta of the tile's 64 queries: one 4-byte DMA per lane, an array per wave.
+      // Entries of queries past the sequence end are never used (block_r masks those queries).
+      if (wave < 3) {
+        const float* src = wave == 0 ? p.taus : (wave == 1 ? p.zinv : p.delta);
+        int qrow = qt * kBN + lane;
+        qrow = qrow < N ? qrow : N - 1;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + q_base + qrow),
+                                         (__attribute__((address_space(3))) void*)&sc[wave][0], 4, 0, 0);
       }
     };
     __syncthreads();
-    int cur = next_tile(t_first - 1);
+    int cur = next_tile(nt);
     if (cur >= 0) issue(a0, b0, c0, scal0, cur);
     while (cur >= 0) {
       __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -571,7 +576,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
                     for (int e = 0; e < 4; ++e) {
                       float pr, u;
                       bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
-                      w[4 * g + e] = pr * zi[e];
+                      w[4 * g + e] = pr > 0.f ? pr * zi[e] : 0.f;
                     }
                   }
                   BT::acc_block(acc, k16 ? ta : doa, qb, w, lq, lh, L - qt * kBN);
