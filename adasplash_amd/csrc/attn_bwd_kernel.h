@@ -426,6 +426,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   __shared__ __align__(1024) unsigned char a1[BT::kNBuf == 2 ? BT::kTile : 16];
   __shared__ __align__(1024) unsigned char b1[BT::kNBuf == 2 ? BT::kTile : 16];
   __shared__ __align__(1024) unsigned char c1[(k16 && BT::kNBuf == 2) ? BT::kTile : 16];
+  // 16-bit types with D <= 64 make one walk over the query tiles and keep both accumulators (at D = 128
+  // the two accumulators plus the K and V fragments no longer fit 256 registers); that needs dO^T and Q^T
+  // at the same time
+  constexpr bool kFused = k16 && D <= 64;
+  __shared__ __align__(1024) unsigned char d0[kFused ? BT::kTile : 16];  // Q^T tile
+  __shared__ __align__(1024) unsigned char d1[(kFused && BT::kNBuf == 2) ? BT::kTile : 16];
   __shared__ __align__(16) float scal0[3][kBN];  // tau, 1 / sum p, delta of the tile's queries
   __shared__ __align__(16) float scal1[3][kBN];
 
@@ -472,9 +478,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     const size_t q_base = (size_t)(b * p.Hq + hq) * N;
     const unsigned char* qg = reinterpret_cast<const unsigned char*>(p.q) + q_base * G::kKRow;
     const unsigned char* dog = reinterpret_cast<const unsigned char*>(p.dout) + q_base * G::kKRow;
+    // transposed operand of the pass: dO^T for dV (pass 1 and the fused pass 3), Q^T for dK (pass 2; the
+    // fused pass takes it as a second transposed tile)
     const unsigned char* tg =
-        k16 ? reinterpret_cast<const unsigned char*>(pass == 1 ? p.dot : p.qt) + (size_t)(b * p.Hq + hq) * D * p.Npad * 2
+        k16 ? reinterpret_cast<const unsigned char*>(pass == 2 ? p.qt : p.dot) + (size_t)(b * p.Hq + hq) * D * p.Npad * 2
             : nullptr;
+    const unsigned char* tg2 =
+        k16 ? reinterpret_cast<const unsigned char*>(p.qt) + (size_t)(b * p.Hq + hq) * D * p.Npad * 2 : nullptr;
     // column of the forward's tile mask for this key block: is any of its two 64-key tiles kept for the
     // 128-row block that holds query tile qt?
     const int32_t* mcol = p.bmask ? p.bmask + (size_t)(b * p.Hq + hq) * p.n_mblk * p.mask_words : nullptr;
@@ -491,10 +501,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
       }
       return -1;
     };
-    auto issue = [&](unsigned char* a, unsigned char* bb, unsigned char* c, float (*sc)[kBN], int qt) {
+    auto issue = [&](unsigned char* a, unsigned char* bb, unsigned char* c, unsigned char* d, float (*sc)[kBN], int qt) {
       BT::issue_rows(qg, qt * kBN, N, a, wave, lane);
-      if (pass == 2 || !k16) BT::issue_rows(dog, qt * kBN, N, bb, wave, lane);
+      if (pass >= 2 || !k16) BT::issue_rows(dog, qt * kBN, N, bb, wave, lane);
       if constexpr (k16) BT::issue_t(tg + (size_t)qt * BT::kTile, c, wave, lane);
+      if constexpr (kFused) {
+        if (pass == 3) BT::issue_t(tg2 + (size_t)qt * BT::kTile, d, wave, lane);
+      }
       // tau, 1 / sum p and delta of the tile's 64 queries: one 4-byte DMA per lane, an array per wave.
       // Entries of queries past the sequence end are never used (block_r masks those queries).
       if (wave < 3) {
@@ -507,19 +520,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     };
     __syncthreads();
     int cur = next_tile(nt);
-    if (cur >= 0) issue(a0, b0, c0, scal0, cur);
+    if (cur >= 0) issue(a0, b0, c0, d0, scal0, cur);
     while (cur >= 0) {
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
       int nxt = next_tile(cur);
       if constexpr (BT::kNBuf == 2) {
-        if (nxt >= 0) issue(a1, b1, c1, scal1, nxt);
+        if (nxt >= 0) issue(a1, b1, c1, d1, scal1, nxt);
         __builtin_amdgcn_sched_barrier(0);
       }
-      body(cur, a0, b0, c0, scal0);
+      body(cur, a0, b0, c0, d0, scal0);
       if constexpr (BT::kNBuf == 1) {
         __syncthreads();
-        if (nxt >= 0) issue(a0, b0, c0, scal0, nxt);
+        if (nxt >= 0) issue(a0, b0, c0, d0, scal0, nxt);
         cur = nxt;
       } else {
         cur = nxt;
@@ -527,9 +540,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
         nxt = next_tile(cur);
-        if (nxt >= 0) issue(a0, b0, c0, scal0, nxt);
+        if (nxt >= 0) issue(a0, b0, c0, d0, scal0, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        body(cur, a1, b1, c1, scal1);
+        body(cur, a1, b1, c1, d1, scal1);
         cur = nxt;
       }
     }
@@ -556,6 +569,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   f32x16 acc[G::kDB];
   unsigned char* stage = (wave < 2 ? a0 : b0) + (wave & 1) * (32 * G::kKRow);
 
+  if constexpr (kFused) {
+    // ---- one walk: dV^T += dO^T P and dK^T += Q^T dX ----
+    f32x16 acc_k[G::kDB];
+#pragma unroll
+    for (int db = 0; db < G::kDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        acc[db][i] = 0.f;
+        acc_k[db][i] = 0.f;
+      }
+    for (int hg = 0; hg < group; ++hg) {
+      tile_loop(kvh * group + hg, 3,
+                [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* dota,
+                    const unsigned char* qta, const float (*sc)[kBN]) {
+#pragma unroll
+                  for (int qb = 0; qb < 2; ++qb) {
+                    if (!block_visible(qt, qb)) continue;
+                    float r[16], w[16];
+                    block_r(qt, qb, qa, sc, r);
+                    // dV first: p / sum p
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                      const f32x4 zi = *reinterpret_cast<const f32x4*>(&sc[1][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+                      for (int e = 0; e < 4; ++e) {
+                        float pr, u;
+                        bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+                        w[4 * g + e] = pr > 0.f ? pr * zi[e] : 0.f;
+                      }
+                    }
+                    BT::acc_block(acc, dota, qb, w, lq, lh, L - qt * kBN);
+                    // then dK: u (dP - delta)
+                    f32x16 dp = BT::dot_block(doa, qb, vf, lq, lh);
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                      const f32x4 di = *reinterpret_cast<const f32x4*>(&sc[2][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+                      for (int e = 0; e < 4; ++e) {
+                        float pr, u;
+                        bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+                        w[4 * g + e] = u > 0.f ? u * (dp[4 * g + e] - di[e]) : 0.f;
+                      }
+                    }
+                    BT::acc_block(acc_k, qta, qb, w, lq, lh, L - qt * kBN);
+                  }
+                });
+    }
+    __syncthreads();
+    BT::store_rows(acc, 1.f, stage, dv_rows, wave_key0, N, lane);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    BT::store_rows(acc_k, p.sm_scale, stage, dk_rows, wave_key0, N, lane);
+    return;
+  }
+
   // ---- pass 1: dV^T += dO^T P ----
 #pragma unroll
   for (int db = 0; db < G::kDB; ++db)
@@ -563,7 +630,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
   for (int hg = 0; hg < group; ++hg) {
     tile_loop(kvh * group + hg, 1,
-              [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const float (*sc)[kBN]) {
+              [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const unsigned char*,
+                  const float (*sc)[kBN]) {
 #pragma unroll
                 for (int qb = 0; qb < 2; ++qb) {
                   if (!block_visible(qt, qb)) continue;
@@ -593,7 +661,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
   for (int hg = 0; hg < group; ++hg) {
     tile_loop(kvh * group + hg, 2,
-              [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const float (*sc)[kBN]) {
+              [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const unsigned char*,
+                  const float (*sc)[kBN]) {
 #pragma unroll
                 for (int qb = 0; qb < 2; ++qb) {
                   if (!block_visible(qt, qb)) continue;
