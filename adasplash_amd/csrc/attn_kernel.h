@@ -416,15 +416,100 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     mask_out[1][i] = 0u;
   }
 
-  // ---- pass A: row max (raw units) ----------------------------------------------------------------------
+  // ---- pass A (+B): row max, and for alpha = 1.5 / 2 the histogram bracket in the same walk ----------------
+  uint32_t* mask_cur = nullptr;  // mask consumed by the next pass
+  uint32_t* mask_new = mask_a;   // mask produced by the running pass
+  const int half = (wave * 32) / kMaskRows;  // which 128-row half of the row block this wave belongs to
+  const bool with_hist = AM != ATT_GEN && p.use_hist;
   float m_raw = -INFINITY;
-  tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
-    for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
+  float hist_lo = 0.f;  // lower bound of tau from the histogram (valid when with_hist)
+  constexpr float kBinW = 1.f / (float)kAttnBins;  // bin width in z units
+  if (!with_hist) {
+    tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
+      for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) m_raw = fmaxf(fmaxf(m_raw, s0[i]), s1[i]);
+        for (int i = 0; i < 16; ++i) m_raw = fmaxf(fmaxf(m_raw, s0[i]), s1[i]);
+      });
     });
-  });
-  m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+    m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+  } else {
+    // The histogram lives on the absolute grid of bins [g / 8, (g + 1) / 8) of z.  A lane counts the bins
+    // g0 .. g0 + 8 with g0 + 8 the bin of the largest score it has met so far, which always covers
+    // [max - 1, max]; whenever that maximum moves up by whole bins the window follows and the bins that
+    // fall off its lower end are dropped (they lie below max - 1 <= tau).  Nine 7-bit counters sit packed
+    // in one 64-bit register (an entry below the window adds to bit 63, which nothing reads) and are
+    // flushed into float counts every third tile.
+    constexpr int W = kAttnBins + 1;
+    constexpr int kNoOrigin = -(1 << 29);
+    const float c8 = (float)kAttnBins * qs;
+    float cnt[W];
+#pragma unroll
+    for (int k = 0; k < W; ++k) cnt[k] = 0.f;
+    unsigned long long packed = 0ull;
+    int since_flush = 0;
+    int g0 = kNoOrigin;
+    auto flush = [&]() {
+#pragma unroll
+      for (int k = 0; k < W; ++k) cnt[k] += (float)((uint32_t)(packed >> (7 * k)) & 0x7fu);
+      packed = 0ull;
+      since_flush = 0;
+    };
+    // moves the window up by sh bins (per lane, sh >= 0): count k takes the place of count k - 1, sh times
+    auto shift_counts = [&](int sh) {
+      sh = sh < W ? sh : W;
+      while (__builtin_amdgcn_ballot_w64(sh > 0) != 0ull) {
+        const bool mv = sh > 0;
+#pragma unroll
+        for (int k = 0; k + 1 < W; ++k) cnt[k] = mv ? cnt[k + 1] : cnt[k];
+        cnt[W - 1] = mv ? 0.f : cnt[W - 1];
+        sh -= mv ? 1 : 0;
+      }
+    };
+    tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
+      bool any = false;
+      for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
+        float tm = m_raw;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tm = fmaxf(fmaxf(tm, s0[i]), s1[i]);
+        m_raw = tm;
+        // bin of the maximum with the same product the entries use (so no entry can land above it)
+        const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : kNoOrigin + kAttnBins;
+        const int sh = g_top - kAttnBins - g0;
+        g0 = g_top - kAttnBins;
+        if (__builtin_amdgcn_ballot_w64(sh > 0) != 0ull) {
+          flush();
+          shift_counts(sh);
+        }
+        const float off = -(float)g0;
+        const unsigned long long before = packed;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+          const float sc = i < 16 ? s0[i & 15] : s1[i & 15];
+          // bins below the window (and the -inf of masked entries) wrap to huge unsigned values
+          const uint32_t idx = (uint32_t)(int)floorf(fmaf(sc, c8, off));
+          const uint32_t slot = idx < (uint32_t)W ? idx : (uint32_t)W;
+          packed += 1ull << __umul24(slot, 7u);
+        }
+        any = ((packed ^ before) << 1) != 0ull;  // some entry of the tile fell inside the window
+      });
+      if (++since_flush == 3) flush();  // <= 32 increments per tile and lane: 3 tiles stay below 128
+      if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
+    });
+    flush();
+    // the two lanes of a row bring their windows to the higher origin and add up
+    const int g0_other = __shfl_xor(g0, 32, 64);
+    const int g0_row = g0 > g0_other ? g0 : g0_other;
+    shift_counts(g0_row - g0);
+#pragma unroll
+    for (int k = 0; k < W; ++k) cnt[k] += __shfl_xor(cnt[k], 32, 64);
+    m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+    // Every entry counts as sitting on the lower edge of its bin, which gives a lower bound of tau that is
+    // less than one bin width off (the entries left out lie below max - 1).
+    const float t_shift = (float)g0_row * kBinW;
+    hist_lo = (AM == ATT_15) ? hist_bracket_alpha15<W>(cnt, t_shift, kBinW) : hist_bracket_alpha2<W>(cnt, t_shift, kBinW);
+    mask_cur = mask_new;
+    mask_new = mask_b;
+  }
   const float m = m_raw * qs;  // row max of z = (alpha-1) q.k / sqrt(D)
 
   // Tightest a-priori bracket: tau in [m - 1, m - n^(1 - alpha)], n = number of valid keys of the row
@@ -434,65 +519,13 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   Bracket br;  // in z units
   br.lo = m - 1.f;
   br.hi = hi_cap;
-  br.t = 0.5f * (br.lo + br.hi);
-
-  uint32_t* mask_cur = nullptr;  // mask consumed by the next pass
-  uint32_t* mask_new = mask_a;   // mask produced by the running pass
-  const int half = (wave * 32) / kMaskRows;  // which 128-row half of the row block this wave belongs to
-
-  // ---- pass B: histogram bracket (alpha = 1.5 or 2) ------------------------------------------------------
-  if (AM != ATT_GEN && p.use_hist) {
-    // Bins are laid on z - t_shift with t_shift a hair below m - 1, so that the rounding differences
-    // between this pass and pass A cannot push the row maximum out of the top bin.
-    const float margin = 1.f / 4096.f;                       // in z units
-    const float t_shift = m - 1.f - margin;
-    const float init = -(m_raw - (1.f + margin) * inv_qs);  // accumulator starts at -t_shift in raw units
-    // the bins span [0, 1 + 2 margin) above t_shift, which puts the maximum (at 1 + margin) inside the top one
-    const float span = 1.f + 2.f * margin;
-    const float c8 = (float)kAttnBins * qs / span;
-    const float bin_w = span / (float)kAttnBins;  // bin width in z units
-    float cnt[kAttnBins];
-#pragma unroll
-    for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] = 0.f;
-    // Nine 7-bit counters in one 64-bit register: slot 0 collects the discarded entries (r < 0; the
-    // float -> uint conversion saturates them to 0), slot 1 + b counts bin b.  An entry that rounding
-    // still lifted past the top edge would shift into bit 63, which nothing reads.
-    unsigned long long packed = 0ull;
-    int since_flush = 0;
-    auto flush = [&]() {
-#pragma unroll
-      for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] += (float)((uint32_t)(packed >> (7 * (bI + 1))) & 0x7fu);
-      packed = 0ull;
-      since_flush = 0;
-    };
-    tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
-      unsigned long long before = packed;
-      for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
-#pragma unroll
-        for (int i = 0; i < 32; ++i) {
-          const float r = i < 16 ? s0[i & 15] : s1[i & 15];
-          const uint32_t slot = (uint32_t)fmaf(r, c8, 1.f);
-          packed += 1ull << __umul24(slot, 7u);
-        }
-      });
-      // a slot above 0 moved <=> some entry of this tile is a candidate (z >= t_shift)
-      const bool any = ((packed ^ before) >> 7) != 0ull;
-      if (++since_flush == 3) flush();  // <= 32 increments per tile and lane: 3 tiles stay below 128
-      if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
-    });
-    flush();
-#pragma unroll
-    for (int bI = 0; bI < kAttnBins; ++bI) cnt[bI] += __shfl_xor(cnt[bI], 32, 64);
-    // Every entry counts as sitting on the lower edge of its bin (the maximum included), which gives a
-    // lower bound lo of tau with tau <= lo + bin width whenever no entry was lost.  The upper end is used
-    // for the starting point only; the bracket keeps the unconditional bound hi_cap.
-    float lo = (AM == ATT_15) ? hist_bracket_alpha15<kAttnBins>(cnt, t_shift, bin_w) : hist_bracket_alpha2<kAttnBins>(cnt, t_shift, bin_w);
-    br.lo = fmaxf(lo - 2e-6f, m - 1.f);
-    br.hi = fminf(br.lo + bin_w + 4e-6f, hi_cap);
-    br.t = 0.5f * (br.lo + br.hi);
-    mask_cur = mask_new;
-    mask_new = mask_b;
+  if (with_hist) {
+    // The nominal upper end lo + bin width serves as the starting point only; pass C replaces it by the
+    // unconditional bound as soon as a Newton step proves it wrong.
+    br.lo = fmaxf(hist_lo - 2e-6f, m - 1.f);
+    br.hi = fminf(br.lo + kBinW + 4e-6f, hi_cap);
   }
+  br.t = 0.5f * (br.lo + br.hi);
 
   // ---- pass C: niter safeguarded Halley / Newton steps ----------------------------------------------------
   {
