@@ -211,43 +211,69 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
 
   // Wave-level load j of a tile fills LDS bytes [1024 j, 1024 j + 1024): chunk position P = 64 j + lane
   // belongs to row P / kC, stored chunk P % kC, i.e. logical chunk (P % kC) ^ sw(row).
-  auto issue_k = [&](unsigned char* kb, int kt) {
+  // Byte offsets of this lane's pieces inside a tile do not depend on the tile: they are kept in registers
+  // and the DMA address is the tile's (wave-uniform) base plus that offset.
+  constexpr int kKPer = (G::kKLoads + NW - 1) / NW, kVPer = (G::kVLoads + NW - 1) / NW;
+  uint32_t koff[kKPer], voff[kVPer];
 #pragma unroll
-    for (int j0 = 0; j0 < (G::kKLoads + NW - 1) / NW; ++j0) {
+  for (int j0 = 0; j0 < kKPer; ++j0) {
+    const int P = (j0 * NW + wave) * 64 + lane;
+    const int row = P / KS::kC;
+    koff[j0] = (uint32_t)(row * G::kKRow + (((P % KS::kC) ^ KS::sw(row)) << 4));
+  }
+#pragma unroll
+  for (int j0 = 0; j0 < kVPer; ++j0) {
+    const int P = (j0 * NW + wave) * 64 + lane;
+    const int row = P / VS::kC;
+    voff[j0] = (uint32_t)(row * G::kVRow + (((P % VS::kC) ^ VS::sw(row)) << 4));
+  }
+  auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKPer], unsigned char* lds, int kt) {
+    // a row-major [64][D] tile out of a row-major tensor (K, or V for fp32); the last tile may stick out
+    const bool whole = (kt + 1) * kBN <= N;
+    const unsigned char* base = g + (size_t)kt * G::kKTile;
+#pragma unroll
+    for (int j0 = 0; j0 < kKPer; ++j0) {
       const int j = j0 * NW + wave;
       if (G::kKLoads % NW == 0 || j < G::kKLoads) {
-        const int P = j * 64 + lane;
-        const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
-        int gk = kt * kBN + row;
-        gk = gk < N ? gk : N - 1;  // rows past the end are masked later; any valid row will do
-        dma16(kglob + (size_t)gk * G::kKRow + c * 16, kb + j * 1024);
-      }
-    }
-  };
-  auto issue_v = [&](unsigned char* vb, int kt) {
-#pragma unroll
-    for (int j0 = 0; j0 < (G::kVLoads + NW - 1) / NW; ++j0) {
-      const int j = j0 * NW + wave;
-      if (G::kVLoads % NW == 0 || j < G::kVLoads) {
-        const int P = j * 64 + lane;
-        const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
-        if constexpr (k16) {
-          dma16(vglob + (size_t)kt * G::kVTile + row * G::kVRow + c * 16, vb + j * 1024);
+        if (whole) {
+          dma16(base + off[j0], lds + j * 1024);
         } else {
+          const int P = j * 64 + lane;
+          const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
           int gk = kt * kBN + row;
-          gk = gk < N ? gk : N - 1;  // p = 0 there
-          dma16(vglob + (size_t)gk * G::kVRow + c * 16, vb + j * 1024);
+          gk = gk < N ? gk : N - 1;  // rows past the end are masked later; any valid row will do
+          dma16(g + (size_t)gk * G::kKRow + c * 16, lds + j * 1024);
         }
       }
     }
   };
+  auto issue_k = [&](unsigned char* kb, int kt) { issue_rows(kglob, koff, kb, kt); };
+  auto issue_v = [&](unsigned char* vb, int kt) {
+    if constexpr (k16) {
+      const unsigned char* base = vglob + (size_t)kt * G::kVTile;  // the transposed copy is padded to whole tiles
+#pragma unroll
+      for (int j0 = 0; j0 < kVPer; ++j0) {
+        const int j = j0 * NW + wave;
+        if (G::kVLoads % NW == 0 || j < G::kVLoads) dma16(base + voff[j0], vb + j * 1024);
+      }
+    } else {
+      issue_rows(vglob, koff, vb, kt);  // same geometry as K
+    }
+  };
 
-  // Next tile index > cur allowed by `mask` (nullptr = every tile), or -1.
+  // Next tile index > cur allowed by `mask` (nullptr = every tile), or -1.  The mask word in use is kept in
+  // a register, so LDS is read once per 32 tiles.
+  int mw_index = -1;
+  uint32_t mw_bits = 0u;
   auto next_tile = [&](const uint32_t* mask, int cur) -> int {
     int t = cur + 1;
     if (!mask) return t < nt ? t : -1;
     while (t < nt) {
-      uint32_t w = mask[t >> 5] >> (t & 31);
+      if ((t >> 5) != mw_index) {
+        mw_index = t >> 5;
+        mw_bits = mask[mw_index];
+      }
+      const uint32_t w = mw_bits >> (t & 31);
       if (w) {
         t += __builtin_ctz(w);
         return t < nt ? t : -1;
@@ -261,6 +287,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   // after the barrier that publishes the current one and completes under the current tile's MFMAs.
   auto tile_loop = [&](const uint32_t* mask, bool with_v, auto&& body) {
     __syncthreads();  // the previous pass is done with the LDS tiles; its mask writes are visible
+    mw_index = -1;
     int cur = next_tile(mask, -1);
     if (cur >= 0) {
       issue_k(k_lds0, cur);
