@@ -473,40 +473,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   const int t_first = p.causal ? n0 / kBN : 0;  // query tiles below the key block see none of its keys
   const int nt = (L + kBN - 1) / kBN;
 
-  // Runs body(qt, tiles, scalars) over the query tiles [t_first, nt) of query head `hq`.
-  auto tile_loop = [&](int hq, int pass, auto&& body) {
-    const size_t q_base = (size_t)(b * p.Hq + hq) * N;
-    const unsigned char* qg = reinterpret_cast<const unsigned char*>(p.q) + q_base * G::kKRow;
-    const unsigned char* dog = reinterpret_cast<const unsigned char*>(p.dout) + q_base * G::kKRow;
-    // transposed operand of the pass: dO^T for dV (pass 1 and the fused pass 3), Q^T for dK (pass 2; the
-    // fused pass takes it as a second transposed tile)
-    const unsigned char* tg =
-        k16 ? reinterpret_cast<const unsigned char*>(pass == 2 ? p.qt : p.dot) + (size_t)(b * p.Hq + hq) * D * p.Npad * 2
-            : nullptr;
-    const unsigned char* tg2 =
-        k16 ? reinterpret_cast<const unsigned char*>(p.qt) + (size_t)(b * p.Hq + hq) * D * p.Npad * 2 : nullptr;
-    // column of the forward's tile mask for this key block: is any of its two 64-key tiles kept for the
-    // 128-row block that holds query tile qt?
-    const int32_t* mcol = p.bmask ? p.bmask + (size_t)(b * p.Hq + hq) * p.n_mblk * p.mask_words : nullptr;
+  // Runs body(qt, tiles, scalars) over every (query tile, query head of the group) pair.  The walk is tile
+  // major and goes from the last tile down: all key blocks of a K/V head then sit on the same query tile at
+  // about the same time, so the workgroups that run side by side on an XCD find the tile in its L2 (head
+  // major, each would soon be streaming another head's tensors and the working set would be all of them).
+  // A step is numbered c = tile * group + head.
+  auto tile_loop = [&](int pass, auto&& body) {
     const int ktile0 = n0 / kBN;
-    auto next_tile = [&](int cur) -> int {
-      // Query tiles are walked from the last one down: every key block of a K/V head then starts on the
-      // same tile and the workgroups that run side by side on an XCD read the same Q / dO tiles at about
-      // the same time, out of its L2 (walking upwards, each would start at its own diagonal).
-      int t = cur - 1;
-      if (!mcol) return t >= t_first ? t : -1;
-      for (; t >= t_first; --t) {
+    auto head_of = [&](int c) { return kvh * group + c % group; };
+    auto next_step = [&](int cur) -> int {
+      int c = cur - 1;
+      if (!p.bmask) return c >= t_first * group ? c : -1;
+      for (; c >= t_first * group; --c) {
+        // column of the forward's tile mask for this key block: is any of its two 64-key tiles kept for
+        // the 128-row block that holds the query tile?  (a 128-key block starts on an even tile, so both
+        // bits sit in one word)
+        const int t = c / group;
+        const int32_t* mcol = p.bmask + (size_t)(b * p.Hq + head_of(c)) * p.n_mblk * p.mask_words;
         const uint32_t w = (uint32_t)mcol[(size_t)(t >> 1) * p.mask_words + (ktile0 >> 5)] >> (ktile0 & 31);
-        if (w & 3u) return t;  // (a 128-key block starts on an even tile, so both bits sit in one word)
+        if (w & 3u) return c;
       }
       return -1;
     };
-    auto issue = [&](unsigned char* a, unsigned char* bb, unsigned char* c, unsigned char* d, float (*sc)[kBN], int qt) {
+    auto issue = [&](unsigned char* a, unsigned char* bb, unsigned char* c, unsigned char* d, float (*sc)[kBN], int step) {
+      const int qt = step / group;
+      const size_t bh = (size_t)(b * p.Hq + head_of(step));
+      const size_t q_base = bh * N;
+      const unsigned char* qg = reinterpret_cast<const unsigned char*>(p.q) + q_base * G::kKRow;
+      const unsigned char* dog = reinterpret_cast<const unsigned char*>(p.dout) + q_base * G::kKRow;
       BT::issue_rows(qg, qt * kBN, N, a, wave, lane);
       if (pass >= 2 || !k16) BT::issue_rows(dog, qt * kBN, N, bb, wave, lane);
-      if constexpr (k16) BT::issue_t(tg + (size_t)qt * BT::kTile, c, wave, lane);
-      if constexpr (kFused) {
-        if (pass == 3) BT::issue_t(tg2 + (size_t)qt * BT::kTile, d, wave, lane);
+      if constexpr (k16) {
+        // transposed operand of the pass: dO^T for dV (pass 1 and the fused pass 3), Q^T for dK (pass 2;
+        // the fused pass takes it as a second transposed tile)
+        const size_t toff = bh * D * p.Npad * 2 + (size_t)qt * BT::kTile;
+        BT::issue_t(reinterpret_cast<const unsigned char*>(pass == 2 ? p.qt : p.dot) + toff, c, wave, lane);
+        if constexpr (kFused) {
+          if (pass == 3) BT::issue_t(reinterpret_cast<const unsigned char*>(p.qt) + toff, d, wave, lane);
+        }
       }
       // tau, 1 / sum p and delta of the tile's 64 queries: one 4-byte DMA per lane, an array per wave.
       // Entries of queries past the sequence end are never used (block_r masks those queries).
@@ -519,17 +523,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
       }
     };
     __syncthreads();
-    int cur = next_tile(nt);
+    int cur = next_step(nt * group);
     if (cur >= 0) issue(a0, b0, c0, d0, scal0, cur);
     while (cur >= 0) {
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
-      int nxt = next_tile(cur);
+      int nxt = next_step(cur);
       if constexpr (BT::kNBuf == 2) {
         if (nxt >= 0) issue(a1, b1, c1, d1, scal1, nxt);
         __builtin_amdgcn_sched_barrier(0);
       }
-      body(cur, a0, b0, c0, d0, scal0);
+      body(cur / group, a0, b0, c0, d0, scal0);
       if constexpr (BT::kNBuf == 1) {
         __syncthreads();
         if (nxt >= 0) issue(a0, b0, c0, d0, scal0, nxt);
@@ -539,10 +543,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
         if (cur < 0) break;
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
-        nxt = next_tile(cur);
+        nxt = next_step(cur);
         if (nxt >= 0) issue(a0, b0, c0, d0, scal0, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        body(cur, a1, b1, c1, d1, scal1);
+        body(cur / group, a1, b1, c1, d1, scal1);
         cur = nxt;
       }
     }
@@ -579,8 +583,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
         acc[db][i] = 0.f;
         acc_k[db][i] = 0.f;
       }
-    for (int hg = 0; hg < group; ++hg) {
-      tile_loop(kvh * group + hg, 3,
+    {
+      tile_loop(3,
                 [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* dota,
                     const unsigned char* qta, const float (*sc)[kBN]) {
 #pragma unroll
@@ -628,8 +632,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   for (int db = 0; db < G::kDB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-  for (int hg = 0; hg < group; ++hg) {
-    tile_loop(kvh * group + hg, 1,
+  {
+    tile_loop(1,
               [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const unsigned char*,
                   const float (*sc)[kBN]) {
 #pragma unroll
@@ -659,8 +663,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   for (int db = 0; db < G::kDB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-  for (int hg = 0; hg < group; ++hg) {
-    tile_loop(kvh * group + hg, 2,
+  {
+    tile_loop(2,
               [&](int qt, const unsigned char* qa, const unsigned char* doa, const unsigned char* ta, const unsigned char*,
                   const float (*sc)[kBN]) {
 #pragma unroll
