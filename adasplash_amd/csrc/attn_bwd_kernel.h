@@ -52,7 +52,7 @@ template <typename T, int D> struct BwdTiles {
   // Double-buffer only while two workgroups still fit a CU: a second resident workgroup hides a tile's
   // load latency better than a second stage does, and brings a second wave to every SIMD.
   static constexpr int kNBuf = (2 * kSlots * kTile <= 64 * 1024) ? 2 : 1;
-  static constexpr int kMinWaves = G::kMinWaves;
+  static constexpr int kMinWaves = G::kMinWaves < 2 ? G::kMinWaves : 2;
   static constexpr int kLoads = kTile / 1024;
 
   // DMA of rows [row0, row0 + 64) of a row-major [N][D] tensor into a swizzled tile.

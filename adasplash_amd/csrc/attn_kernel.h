@@ -80,8 +80,10 @@ template <typename T, int D> struct TileGeo {
   static constexpr int kNW = 4;
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
-  // shapes whose live state fits 256 registers are held to two waves per SIMD; the others take what they need
-  static constexpr int kMinWaves = ((k16 && D <= 128) || (!k16 && D <= 64)) ? 2 : 1;
+  // Waves per SIMD the register allocation is held to.  The walks are bound by dependent latency, so more
+  // resident waves pay even at the price of a few spills: four for 16-bit D <= 64 (C5 23.3 -> 16.3 ms),
+  // two where the live state needs up to 256 registers, one for the shapes that need more.
+  static constexpr int kMinWaves = (k16 && D <= 64) ? 4 : (((k16 && D <= 128) || (!k16 && D <= 64)) ? 2 : 1);
   static constexpr int kQRegs = k16 ? (D / 16) * 4 : D / 2;  // dwords of Q held per lane
   static constexpr int kDB = D >= 32 ? D / 32 : 1;           // 32-wide d blocks of the output
   static constexpr int kKLoads = kKTile / 1024;              // wave-level 1 KB DMA instructions per K tile
@@ -100,7 +102,7 @@ template <int AM> __device__ __forceinline__ float attn_prob(float r, float qs, 
 }
 
 template <typename T, int D, int AM>
-__global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_waves_per_eu(TileGeo<T, D>::kMinWaves, 2))) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_waves_per_eu(TileGeo<T, D>::kMinWaves, (TileGeo<T, D>::kMinWaves > 2 ? TileGeo<T, D>::kMinWaves : 2)))) void attn_fwd_kernel(AttnParams p) {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
   using VS = Swz<G::kVRow>;
