@@ -36,6 +36,27 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+// per 16-bit half: v >> sh, 1 << slot
+__device__ __forceinline__ uint32_t pk_shr16(uint32_t v, uint32_t sh2) {
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2_t, v) >> __builtin_bit_cast(u16x2_t, sh2));
+}
+__device__ __forceinline__ uint32_t pk_onehot16(uint32_t slot2) {
+  const u16x2_t one = {1, 1};
+  return __builtin_bit_cast(uint32_t, one << __builtin_bit_cast(u16x2_t, slot2));
+}
+// bitwise full adder: a + b + c = sum + 2 carry
+__device__ __forceinline__ void full_add(uint32_t a, uint32_t b, uint32_t c, uint32_t& sum, uint32_t& carry) {
+  // one three-input bit operation each (truth tables of xor3 and majority)
+  const uint32_t x = __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+  carry = __builtin_amdgcn_bitop3_b32(a, b, c, 0xe8);
+  sum = x;
+}
+
+// two floats -> packed f16, rounded towards zero (one instruction)
+__device__ __forceinline__ h2_t pkrtz(float a, float b) { return __builtin_bit_cast(h2_t, __builtin_amdgcn_cvt_pkrtz(a, b)); }
 
 template <typename T> struct is16 { static constexpr bool value = true; };
 template <> struct is16<float> { static constexpr bool value = false; };
@@ -51,8 +72,16 @@ template <> __device__ __forceinline__ f32x16 mfma_16bit<f16_t>(u32x4 a, u32x4 b
 // 16-byte global -> LDS copy per lane: lane i of the wave writes LDS bytes [16 i, 16 i + 16) after the
 // wave-uniform base `lds`, from its own global address.
 __device__ __forceinline__ void dma16(const void* gsrc, void* lds) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+  // Issued as inline assembly on purpose: the compiler treats the builtin form as an access that may touch both
+  // memory and LDS, and while one is in flight it waits for *every* outstanding LDS read (lgkmcnt(0)) before the
+  // first use of any of them.  The hardware does not count this load in lgkmcnt (measured), so the tile loop's
+  // own vmcnt(0) + barrier is all the ordering it needs; the "memory" clobber keeps LDS accesses from moving
+  // across it.
+  const uint32_t base = (uint32_t)(uintptr_t)lds;  // wave-uniform LDS byte address
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane(base))
+               : "memory", "m0");
 }
 
 // Tile geometry.  A tile row has kC 16-byte chunks; chunk c of row r is stored at chunk position
@@ -414,12 +443,16 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     if (p.causal && kt * kBN > wave_row0 + 31) return;
     const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
     f32x16 s0, s1;
+    // The two arms start with distinct fences so that their common LDS reads are not hoisted above the branch:
+    // reads and MFMAs then share a basic block and the reads are waited for one by one, not all at once.
     if (need_mask) {
+      asm volatile("; masked tile" ::: "memory");
       tile_scores(kt_lds, init, s0, s1);
       mask_block(s0, kt, 0);
       mask_block(s1, kt, 1);
       f(s0, s1);
     } else {
+      asm volatile("; plain tile" ::: "memory");
       tile_scores(kt_lds, init, s0, s1);
       f(s0, s1);
     }
@@ -465,34 +498,30 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     // The histogram lives on the absolute grid of bins [g / 8, (g + 1) / 8) of z.  A lane counts the bins
     // g0 .. g0 + 8 with g0 + 8 the bin of the largest score it has met so far, which always covers
     // [max - 1, max]; whenever that maximum moves up by whole bins the window follows and the bins that
-    // fall off its lower end are dropped (they lie below max - 1 <= tau).  Nine 7-bit counters sit packed
-    // in one 64-bit register (an entry below the window adds to bit 63, which nothing reads) and are
-    // flushed into float counts every third tile.
+    // fall off its lower end are dropped (they lie below max - 1 <= tau).
+    //
+    // Counting is bit-sliced.  Two scores become one 32-bit word of two one-hot 16-bit halves -- bit b + 1 for
+    // window bin b, bit 0 for everything below the window -- in 2 instructions per score (an fma to window
+    // coordinates, a saturating float -> u16 pair conversion, a packed shift).  The 16 words of a tile go
+    // through a carry-save adder tree (3-input xor / majority, 1 instruction per score) into bit planes:
+    // plane k holds bit k of every counter, so a lane keeps 2 x 10 counters of kPlanes bits in kPlanes
+    // registers.  Moving the window is one packed shift per plane.
     constexpr int W = kAttnBins + 1;
     constexpr int kNoOrigin = -(1 << 29);
+    constexpr int kPlanes = 20;  // a lane meets every other key of its row: up to 2^19 with the 1M-key mask
+    constexpr uint32_t kBinBits = 0xfffefffeu;  // everything but the below-window bit of each half
     const float c8 = (float)kAttnBins * qs;
-    float cnt[W];
+    const float c8n = c8 * (1.f / 65535.f);  // the conversion maps [0, 1] to [0, 65535] and rounds to nearest
+    uint32_t pl[kPlanes];
 #pragma unroll
-    for (int k = 0; k < W; ++k) cnt[k] = 0.f;
-    unsigned long long packed = 0ull;
-    int since_flush = 0;
+    for (int k = 0; k < kPlanes; ++k) pl[k] = 0u;
     int g0 = kNoOrigin;
-    auto flush = [&]() {
+    // moves the window up by sh bins (per lane, sh >= 0)
+    auto shift_planes = [&](int sh) {
+      const uint32_t s1 = (uint32_t)(sh < 15 ? sh : 15);
+      const uint32_t s2 = s1 | (s1 << 16);
 #pragma unroll
-      for (int k = 0; k < W; ++k) cnt[k] += (float)((uint32_t)(packed >> (7 * k)) & 0x7fu);
-      packed = 0ull;
-      since_flush = 0;
-    };
-    // moves the window up by sh bins (per lane, sh >= 0): count k takes the place of count k - 1, sh times
-    auto shift_counts = [&](int sh) {
-      sh = sh < W ? sh : W;
-      while (__builtin_amdgcn_ballot_w64(sh > 0) != 0ull) {
-        const bool mv = sh > 0;
-#pragma unroll
-        for (int k = 0; k + 1 < W; ++k) cnt[k] = mv ? cnt[k + 1] : cnt[k];
-        cnt[W - 1] = mv ? 0.f : cnt[W - 1];
-        sh -= mv ? 1 : 0;
-      }
+      for (int k = 0; k < kPlanes; ++k) pl[k] = pk_shr16(pl[k], s2);
     };
     tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
       bool any = false;
@@ -501,34 +530,73 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
 #pragma unroll
         for (int i = 0; i < 16; ++i) tm = fmaxf(fmaxf(tm, s0[i]), s1[i]);
         m_raw = tm;
-        // bin of the maximum with the same product the entries use (so no entry can land above it)
+        // bin of the maximum; the entries use the same scale, so none lands more than a rounding error above it
         const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : kNoOrigin + kAttnBins;
         const int sh = g_top - kAttnBins - g0;
         g0 = g_top - kAttnBins;
-        if (__builtin_amdgcn_ballot_w64(sh > 0) != 0ull) {
-          flush();
-          shift_counts(sh);
-        }
-        const float off = -(float)g0;
-        const unsigned long long before = packed;
+        if (__builtin_amdgcn_ballot_w64(sh > 0) != 0ull) shift_planes(sh);
+        // window coordinate y = s c8 - g0 + 1: [0, 1) below the window, [b + 1, b + 2) in bin b; the conversion
+        // rounds, hence the half
+        const float offn = (0.5f - (float)g0) * (1.f / 65535.f);
+        uint32_t w[16];
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-          const float sc = i < 16 ? s0[i & 15] : s1[i & 15];
-          // bins below the window (and the -inf of masked entries) wrap to huge unsigned values
-          const uint32_t idx = (uint32_t)(int)floorf(fmaf(sc, c8, off));
-          const uint32_t slot = idx < (uint32_t)W ? idx : (uint32_t)W;
-          packed += 1ull << __umul24(slot, 7u);
+        for (int j = 0; j < 16; ++j) {
+          const float sa = j < 8 ? s0[(2 * j) & 15] : s1[(2 * j) & 15];
+          const float sb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
+          w[j] = pk_onehot16(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_u16(fmaf(sa, c8n, offn), fmaf(sb, c8n, offn))));
         }
-        any = ((packed ^ before) << 1) != 0ull;  // some entry of the tile fell inside the window
+        uint32_t seen = 0u;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) seen |= w[j];
+        any = (seen & kBinBits) != 0u;  // some entry of the tile fell inside the window
+        // adder tree: 16 words + plane 0 -> plane 0 and 8 carries, those + plane 1 -> plane 1 and 4 carries, ...
+        uint32_t c2[8], c4[4], c8w[2], c16;
+        uint32_t acc = pl[0];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) full_add(acc, w[2 * j], w[2 * j + 1], acc, c2[j]);
+        pl[0] = acc;
+        acc = pl[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) full_add(acc, c2[2 * j], c2[2 * j + 1], acc, c4[j]);
+        pl[1] = acc;
+        acc = pl[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) full_add(acc, c4[2 * j], c4[2 * j + 1], acc, c8w[j]);
+        pl[2] = acc;
+        acc = pl[3];
+        full_add(acc, c8w[0], c8w[1], acc, c16);
+        pl[3] = acc;
+        // the carry out of the tree ripples through the upper planes; the below-window bit would carry on
+        // every tile and is dropped
+        uint32_t carry = c16 & kBinBits;
+#pragma unroll
+        for (int k = 4; k < kPlanes; ++k) {
+          if (__builtin_amdgcn_ballot_w64(carry != 0u) == 0ull) break;
+          const uint32_t t = pl[k] & carry;
+          pl[k] ^= carry;
+          carry = t;
+        }
       });
-      if (++since_flush == 3) flush();  // <= 32 increments per tile and lane: 3 tiles stay below 128
       if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
     });
-    flush();
-    // the two lanes of a row bring their windows to the higher origin and add up
+    // the two lanes of a row bring their windows to the higher origin; then the counters are read out of the
+    // planes (both halves of a word belong to the lane's row) and added up
     const int g0_other = __shfl_xor(g0, 32, 64);
     const int g0_row = g0 > g0_other ? g0 : g0_other;
-    shift_counts(g0_row - g0);
+    shift_planes(g0_row - g0);
+    float cnt[W];
+#pragma unroll
+    for (int bin = 0; bin < W; ++bin) {
+      uint32_t c = 0u;
+#pragma unroll
+      for (int k = 0; k < kPlanes; ++k) {
+        uint32_t bits = ((pl[k] >> (bin + 1)) & 1u) + ((pl[k] >> (bin + 17)) & 1u);
+        // an entry a rounding error above the top bin counts as sitting in it
+        if (bin == W - 1) bits += ((pl[k] >> (bin + 2)) & 1u) + ((pl[k] >> (bin + 18)) & 1u);
+        c += bits << k;
+      }
+      cnt[bin] = (float)c;
+    }
 #pragma unroll
     for (int k = 0; k < W; ++k) cnt[k] += __shfl_xor(cnt[k], 32, 64);
     m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
@@ -551,7 +619,8 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   if (with_hist) {
     // The nominal upper end lo + bin width serves as the starting point only; pass C replaces it by the
     // unconditional bound as soon as a Newton step proves it wrong.
-    br.lo = fmaxf(hist_lo - 2e-6f, m - 1.f);
+    // the margin covers the rounding of the window coordinates (relative 2^-23 of the score's magnitude)
+    br.lo = fmaxf(hist_lo - (2e-6f + 5e-7f * fabsf(m)), m - 1.f);
     br.hi = fminf(br.lo + kBinW + 4e-6f, hi_cap);
   }
   br.t = 0.5f * (br.lo + br.hi);
@@ -564,9 +633,36 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       const float dl = (br.lo - br.t) * inv_qs;  // z > lo  <=>  (s - t_raw) > dl
       const bool refine = true;  // every step tightens the tile mask to {z > lower bound} for the next pass
       float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-      int cnt_pos = 0;
+      int cnt_pos = 0, cnt_neg = 0, n_seen = 0;  // n_seen - cnt_neg: scores above the threshold (packed path)
       tile_loop(mask_cur, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
         float dmax = -INFINITY;
+        if constexpr (k16 && AM != ATT_GEN) {
+          // 16-bit inputs: the sums run on pairs of scores rounded (towards zero) to f16 -- packed max, two-term
+          // dot products with fp32 accumulation, and the sign bits for the support count: 3.5 VALU
+          // instructions per score instead of 5.5.  The rounding moves f by a few 1e-4 relative, far inside
+          // the 16-bit output tolerance, and keeps {score > lower bound} a superset (negative values round up).
+          h2_t dm2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+          const h2_t zero2 = {(_Float16)0.f, (_Float16)0.f}, one2 = {(_Float16)1.f, (_Float16)1.f};
+          for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
+            n_seen += 32;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+              const float ra = j < 8 ? s0[(2 * j) & 15] : s1[(2 * j) & 15];
+              const float rb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
+              const h2_t h = pkrtz(ra, rb);
+              dm2 = __builtin_elementwise_max(dm2, h);
+              cnt_neg += __builtin_popcount(__builtin_bit_cast(uint32_t, h) & 0x80008000u);
+              const h2_t u = __builtin_elementwise_max(h, zero2);
+              if constexpr (AM == ATT_15) {
+                a0 = __builtin_amdgcn_fdot2(u, u, a0, false);
+                a1 = __builtin_amdgcn_fdot2(u, one2, a1, false);
+              } else {
+                a0 = __builtin_amdgcn_fdot2(u, one2, a0, false);
+              }
+            }
+          });
+          dmax = fmaxf((float)dm2[0], (float)dm2[1]);
+        } else {
         for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
           if (refine) {
 #pragma unroll
@@ -596,8 +692,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
             }
           }
         });
+        }
         if (refine && __builtin_amdgcn_ballot_w64(dmax > dl) != 0ull && lane == 0) mark_tile(mask_new, kt);
       });
+      if constexpr (k16 && AM != ATT_GEN) cnt_pos = n_seen - cnt_neg;
       if constexpr (AM == ATT_15) {
         a0 *= qs * qs;
         a1 *= qs;
