@@ -39,13 +39,12 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
 typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
-// per 16-bit half: v >> sh, 1 << slot
+// per 16-bit half: v >> sh, v << sh
 __device__ __forceinline__ uint32_t pk_shr16(uint32_t v, uint32_t sh2) {
   return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2_t, v) >> __builtin_bit_cast(u16x2_t, sh2));
 }
-__device__ __forceinline__ uint32_t pk_onehot16(uint32_t slot2) {
-  const u16x2_t one = {1, 1};
-  return __builtin_bit_cast(uint32_t, one << __builtin_bit_cast(u16x2_t, slot2));
+__device__ __forceinline__ uint32_t pk_shl16(uint32_t v, uint32_t sh2) {
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2_t, v) << __builtin_bit_cast(u16x2_t, sh2));
 }
 // bitwise full adder: a + b + c = sum + 2 carry
 __device__ __forceinline__ void full_add(uint32_t a, uint32_t b, uint32_t c, uint32_t& sum, uint32_t& carry) {
@@ -260,15 +259,18 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   }
   auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKPer], unsigned char* lds, int kt) {
     // a row-major [64][D] tile out of a row-major tensor (K, or V for fp32); the last tile may stick out
-    const bool whole = (kt + 1) * kBN <= N;
     const unsigned char* base = g + (size_t)kt * G::kKTile;
+    if ((kt + 1) * kBN <= N) {  // one branch per tile, then straight-line loads
 #pragma unroll
-    for (int j0 = 0; j0 < kKPer; ++j0) {
-      const int j = j0 * NW + wave;
-      if (G::kKLoads % NW == 0 || j < G::kKLoads) {
-        if (whole) {
-          dma16(base + off[j0], lds + j * 1024);
-        } else {
+      for (int j0 = 0; j0 < kKPer; ++j0) {
+        const int j = j0 * NW + wave;
+        if (G::kKLoads % NW == 0 || j < G::kKLoads) dma16(base + off[j0], lds + j * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int j0 = 0; j0 < kKPer; ++j0) {
+        const int j = j0 * NW + wave;
+        if (G::kKLoads % NW == 0 || j < G::kKLoads) {
           const int P = j * 64 + lane;
           const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
           int gk = kt * kBN + row;
@@ -495,20 +497,23 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     });
     m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
   } else {
-    // The histogram lives on the absolute grid of bins [g / 8, (g + 1) / 8) of z.  A lane counts the bins
-    // g0 .. g0 + 8 with g0 + 8 the bin of the largest score it has met so far, which always covers
-    // [max - 1, max]; whenever that maximum moves up by whole bins the window follows and the bins that
-    // fall off its lower end are dropped (they lie below max - 1 <= tau).
+    // The histogram lives on the absolute grid of bins [g / 8, (g + 1) / 8) of z; the solver needs the nine bins
+    // g_top - 8 .. g_top below the bin of the row maximum, which cover [max - 1, max] (everything lower is
+    // below tau).  A lane counts the 15 bins g0 .. g0 + 14 and keeps the bin of its running maximum among the
+    // upper seven of them: only when the maximum climbs past the window does the window move (up to the
+    // point where the maximum sits in its ninth bin again), dropping the bins that fall off the lower end.
     //
-    // Counting is bit-sliced.  Two scores become one 32-bit word of two one-hot 16-bit halves -- bit b + 1 for
-    // window bin b, bit 0 for everything below the window -- in 2 instructions per score (an fma to window
+    // Counting is bit-sliced.  Two scores become one 32-bit word of two one-hot 16-bit halves -- bit g - g0 + 1
+    // for bin g, bit 0 for everything below the window -- in 2 instructions per score (an fma to window
     // coordinates, a saturating float -> u16 pair conversion, a packed shift).  The 16 words of a tile go
     // through a carry-save adder tree (3-input xor / majority, 1 instruction per score) into bit planes:
-    // plane k holds bit k of every counter, so a lane keeps 2 x 10 counters of kPlanes bits in kPlanes
+    // plane k holds bit k of every counter, so a lane keeps 2 x 15 counters of kPlanes bits in kPlanes
     // registers.  Moving the window is one packed shift per plane.
     constexpr int W = kAttnBins + 1;
     constexpr int kNoOrigin = -(1 << 29);
-    constexpr int kPlanes = 20;  // a lane meets every other key of its row: up to 2^19 with the 1M-key mask
+    constexpr int kPlanes = 20;     // a lane meets every other key of its row: up to 2^19 with the 1M-key mask
+    constexpr int kRipple = 9;      // planes below this one take the tile's carry unconditionally
+    constexpr int kTopLo = W, kTopHi = 15;      // bit positions the bin of the maximum may occupy
     constexpr uint32_t kBinBits = 0xfffefffeu;  // everything but the below-window bit of each half
     const float c8 = (float)kAttnBins * qs;
     const float c8n = c8 * (1.f / 65535.f);  // the conversion maps [0, 1] to [0, 65535] and rounds to nearest
@@ -516,6 +521,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
 #pragma unroll
     for (int k = 0; k < kPlanes; ++k) pl[k] = 0u;
     int g0 = kNoOrigin;
+    // window coordinate y = s c8 - g0 + 1: [0, 1) below the window, [i, i + 1) at bit position i; the
+    // conversion rounds, hence the half
+    float offn = (0.5f - (float)g0) * (1.f / 65535.f);
+    uint32_t live2 = 0u;  // bit positions of the nine bins under the running maximum, in both halves
     // moves the window up by sh bins (per lane, sh >= 0)
     auto shift_planes = [&](int sh) {
       const uint32_t s1 = (uint32_t)(sh < 15 ? sh : 15);
@@ -531,24 +540,30 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
         for (int i = 0; i < 16; ++i) tm = fmaxf(fmaxf(tm, s0[i]), s1[i]);
         m_raw = tm;
         // bin of the maximum; the entries use the same scale, so none lands more than a rounding error above it
-        const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : kNoOrigin + kAttnBins;
-        const int sh = g_top - kAttnBins - g0;
-        g0 = g_top - kAttnBins;
-        if (__builtin_amdgcn_ballot_w64(sh > 0) != 0ull) shift_planes(sh);
-        // window coordinate y = s c8 - g0 + 1: [0, 1) below the window, [b + 1, b + 2) in bin b; the conversion
-        // rounds, hence the half
-        const float offn = (0.5f - (float)g0) * (1.f / 65535.f);
+        const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : g0 + kTopLo - 1;
+        int p_top = g_top - g0 + 1;
+        if (__builtin_amdgcn_ballot_w64(p_top > kTopHi) != 0ull) {
+          const int sh = p_top > kTopHi ? p_top - kTopLo : 0;
+          shift_planes(sh);
+          g0 += sh;
+          p_top -= sh;
+          offn = (0.5f - (float)g0) * (1.f / 65535.f);
+        }
+        {
+          const uint32_t lo = (uint32_t)(p_top - kAttnBins);
+          live2 = pk_shl16(0xffffffffu, lo | (lo << 16));
+        }
         uint32_t w[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
           const float sa = j < 8 ? s0[(2 * j) & 15] : s1[(2 * j) & 15];
           const float sb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
-          w[j] = pk_onehot16(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_u16(fmaf(sa, c8n, offn), fmaf(sb, c8n, offn))));
+          w[j] = pk_shl16(0x00010001u, __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_u16(fmaf(sa, c8n, offn), fmaf(sb, c8n, offn))));
         }
         uint32_t seen = 0u;
 #pragma unroll
         for (int j = 0; j < 16; ++j) seen |= w[j];
-        any = (seen & kBinBits) != 0u;  // some entry of the tile fell inside the window
+        any = (seen & live2) != 0u;  // some entry of the tile lies within 1 of the running maximum
         // adder tree: 16 words + plane 0 -> plane 0 and 8 carries, those + plane 1 -> plane 1 and 4 carries, ...
         uint32_t c2[8], c4[4], c8w[2], c16;
         uint32_t acc = pl[0];
@@ -566,24 +581,31 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
         acc = pl[3];
         full_add(acc, c8w[0], c8w[1], acc, c16);
         pl[3] = acc;
-        // the carry out of the tree ripples through the upper planes; the below-window bit would carry on
-        // every tile and is dropped
+        // the carry out of the tree ripples through the next planes; a carry into plane kRipple is rare enough
+        // for a branch.  The below-window bit would carry on every tile and is dropped.
         uint32_t carry = c16 & kBinBits;
 #pragma unroll
-        for (int k = 4; k < kPlanes; ++k) {
-          if (__builtin_amdgcn_ballot_w64(carry != 0u) == 0ull) break;
+        for (int k = 4; k < kRipple; ++k) {
           const uint32_t t = pl[k] & carry;
           pl[k] ^= carry;
           carry = t;
         }
+        if (__builtin_amdgcn_ballot_w64(carry != 0u) != 0ull) {
+#pragma unroll
+          for (int k = kRipple; k < kPlanes; ++k) {
+            const uint32_t t = pl[k] & carry;
+            pl[k] ^= carry;
+            carry = t;
+          }
+        }
       });
       if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
     });
-    // the two lanes of a row bring their windows to the higher origin; then the counters are read out of the
-    // planes (both halves of a word belong to the lane's row) and added up
-    const int g0_other = __shfl_xor(g0, 32, 64);
-    const int g0_row = g0 > g0_other ? g0 : g0_other;
-    shift_planes(g0_row - g0);
+    // the two lanes of a row bring their windows to the row's nine bins, bin g_top - 8 at bit position 1; then
+    // the counters are read out of the planes (both halves of a word belong to the lane's row) and added up
+    m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+    const int g0_row = (m_raw > -INFINITY ? (int)floorf(m_raw * c8) : kNoOrigin + kAttnBins) - kAttnBins;
+    shift_planes(g0_row - g0);  // >= 0: a lane's window starts at or below its own maximum's ninth bin
     float cnt[W];
 #pragma unroll
     for (int bin = 0; bin < W; ++bin) {
@@ -599,7 +621,6 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     }
 #pragma unroll
     for (int k = 0; k < W; ++k) cnt[k] += __shfl_xor(cnt[k], 32, 64);
-    m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
     // Every entry counts as sitting on the lower edge of its bin, which gives a lower bound of tau that is
     // less than one bin width off (the entries left out lie below max - 1).
     const float t_shift = (float)g0_row * kBinW;
@@ -625,6 +646,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   }
   br.t = 0.5f * (br.lo + br.hi);
 
+#if defined(ADSP_EXP_STOP) && ADSP_EXP_STOP == 1
+  if (p.taus && qi < L && lh == 0) p.taus[(size_t)(b * p.Hq + h) * N + qi] = br.t + hist_lo;
+  return;
+#endif
   // ---- pass C: niter safeguarded Halley / Newton steps ----------------------------------------------------
   {
     float t_prev = br.t, f_prev = 0.f;
@@ -723,6 +748,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   }
   const float tau = br.t;
 
+#if defined(ADSP_EXP_STOP) && ADSP_EXP_STOP == 2
+  if (p.taus && qi < L && lh == 0) p.taus[(size_t)(b * p.Hq + h) * N + qi] = br.t;
+  return;
+#endif
   // ---- pass D: out = sum_j p_j v_j / sum_j p_j over the masked tiles --------------------------------------
   f32x16 o[G::kDB];
 #pragma unroll
