@@ -358,7 +358,7 @@ template <typename T, int AM> __global__ __launch_bounds__(256) void entmax_rows
       s[1] += u;
     }
     row_sum<256, 2>(s, sm);
-    const float q = s[0] / s[1];
+    const float q = s[1] > 0.f ? s[0] / s[1] : 0.f;
     for (long long j = threadIdx.x; j < cols; j += 256) {
       float yy = load_elem<T>(y, base + j);
       float g = load_elem<T>(dy, base + j);
@@ -367,6 +367,83 @@ template <typename T, int AM> __global__ __launch_bounds__(256) void entmax_rows
       store_elem<T>(dx, base + j, u * g - q * u);
     }
     __syncthreads();
+  }
+}
+
+// Register-resident backward: y and dy are read from HBM once (16-byte non-temporal loads), dx is written
+// once.  The support of an entmax row is small, so most 16-byte chunks of y are all zeros: their dy is never
+// loaded and their dx is stored as zeros without arithmetic.
+template <int AM> __device__ __forceinline__ float bwd_u(float yy, float cf) {
+  if (!(yy > 0.f)) return 0.f;
+  if constexpr (AM == AM_2) return 1.f;
+  if constexpr (AM == AM_15) return __builtin_amdgcn_sqrtf(yy);  // one instruction, 1 ulp
+  return fast_exp2(fast_log2(fmaxf(yy, 1e-6f)) * cf);
+}
+
+template <typename T, int AM, int NCHUNK, int TPR>
+__global__ __launch_bounds__(256) void entmax_rows_bwd_reg_kernel(const void* y, const void* dy, void* dx,
+                                                                     long long rows, long long cols, float cf) {
+  constexpr int kVec = elem_traits<T>::kVec;
+  constexpr int kRowsPerBlock = 256 / TPR;
+  __shared__ float sm[32];
+  const int tid = threadIdx.x;
+  const int t_in_row = tid % TPR, r_in_blk = tid / TPR;
+  const long long row = (long long)blockIdx.x * kRowsPerBlock + r_in_blk;
+  if (row >= rows) return;  // TPR == 256: the whole block; TPR == 64: a wave, and no block barrier is used
+  const long long nvec = cols / kVec;
+  const size_t row_bytes = (size_t)row * cols * elem_traits<T>::kBytes;
+  const u32x4* yrow = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(y) + row_bytes);
+  const u32x4* grow = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(dy) + row_bytes);
+  u32x4* xrow = reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dx) + row_bytes);
+
+  u32x4 yr[NCHUNK], gr[NCHUNK];
+  bool valid[NCHUNK], live[NCHUNK];
+  // every lane loads (a lane past the row end re-reads the row's last chunk and ignores it): no branches, so
+  // all the loads of a row are in flight together
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const long long vi = (long long)c * TPR + t_in_row;
+    valid[c] = vi < nvec;
+    yr[c] = __builtin_nontemporal_load(yrow + (valid[c] ? vi : nvec - 1));
+  }
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) live[c] = valid[c] && (yr[c][0] | yr[c][1] | yr[c][2] | yr[c][3]) != 0u;
+  // dy matters only where y has a non-zero element: the other lanes re-read the row's first chunk (one cached
+  // line per wave instead of a kilobyte of HBM traffic) so that these loads need no branch either
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) gr[c] = __builtin_nontemporal_load(grow + (live[c] ? (long long)c * TPR + t_in_row : 0ll));
+  float s[2] = {0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    if (live[c]) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const float u = bwd_u<AM>(chunk_elem<T>(yr[c], e), cf);
+        s[0] = fmaf(u, chunk_elem<T>(gr[c], e), s[0]);
+        s[1] += u;
+      }
+    }
+  }
+  row_sum<TPR, 2>(s, sm);
+  const float q = s[1] > 0.f ? s[0] / s[1] : 0.f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    if (valid[c]) {
+      u32x4 o = {0u, 0u, 0u, 0u};
+      if (live[c]) {
+        if constexpr (kVec == 4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = __builtin_bit_cast(uint32_t, bwd_u<AM>(chunk_elem<T>(yr[c], e), cf) * (chunk_elem<T>(gr[c], e) - q));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = pack2<T>(bwd_u<AM>(chunk_elem<T>(yr[c], 2 * e), cf) * (chunk_elem<T>(gr[c], 2 * e) - q),
+                            bwd_u<AM>(chunk_elem<T>(yr[c], 2 * e + 1), cf) * (chunk_elem<T>(gr[c], 2 * e + 1) - q));
+        }
+      }
+      __builtin_nontemporal_store(o, xrow + (long long)c * TPR + t_in_row);
+    }
   }
 }
 
@@ -414,8 +491,37 @@ template <typename T> static void launch_fwd_am(const RowsParams& p, int am, boo
   return launch_fwd<T, AM_GEN>(p, aligned, force_tpr, s);
 }
 
+template <typename T, int AM, int NCHUNK, int TPR>
+static void launch_bwd_reg(const void* y, const void* dy, void* dx, long long rows, long long cols, float cf, hipStream_t s) {
+  constexpr int rpb = 256 / TPR;
+  const long long blocks = (rows + rpb - 1) / rpb;
+  hipLaunchKernelGGL((entmax_rows_bwd_reg_kernel<T, AM, NCHUNK, TPR>), dim3((unsigned)blocks), dim3(256), 0, s, y, dy, dx,
+                     rows, cols, cf);
+}
+
+// true if a register-resident kernel took the row shape
+template <typename T, int AM>
+static bool launch_bwd_fast(const void* y, const void* dy, void* dx, long long rows, long long cols, float cf, hipStream_t s) {
+  constexpr int kVec = elem_traits<T>::kVec;
+  const bool aligned = (((uintptr_t)y | (uintptr_t)dy | (uintptr_t)dx) & 15) == 0;
+  if (!aligned || cols % kVec != 0 || rows >= (1ll << 31)) return false;
+  const long long nvec = cols / kVec;
+  const long long c64 = (nvec + 63) / 64, c256 = (nvec + 255) / 256;
+  if (c64 <= 1) return launch_bwd_reg<T, AM, 1, 64>(y, dy, dx, rows, cols, cf, s), true;
+  if (c64 <= 2) return launch_bwd_reg<T, AM, 2, 64>(y, dy, dx, rows, cols, cf, s), true;
+  if (c64 <= 4) return launch_bwd_reg<T, AM, 4, 64>(y, dy, dx, rows, cols, cf, s), true;
+  if (c256 <= 2) return launch_bwd_reg<T, AM, 2, 256>(y, dy, dx, rows, cols, cf, s), true;
+  if (c256 <= 4) return launch_bwd_reg<T, AM, 4, 256>(y, dy, dx, rows, cols, cf, s), true;
+  if (c256 <= 8) return launch_bwd_reg<T, AM, 8, 256>(y, dy, dx, rows, cols, cf, s), true;
+  if (c256 <= 16) return launch_bwd_reg<T, AM, 16, 256>(y, dy, dx, rows, cols, cf, s), true;
+  return false;
+}
+
 template <typename T> static void launch_bwd_am(const void* y, const void* dy, void* dx, long long rows, long long cols,
                                                 int am, float cf, hipStream_t s) {
+  if (am == AM_15 && launch_bwd_fast<T, AM_15>(y, dy, dx, rows, cols, cf, s)) return;
+  if (am == AM_2 && launch_bwd_fast<T, AM_2>(y, dy, dx, rows, cols, cf, s)) return;
+  if (am == AM_GEN && launch_bwd_fast<T, AM_GEN>(y, dy, dx, rows, cols, cf, s)) return;
   long long blocks = rows < 65536 ? rows : 65536;
   if (am == AM_15)
     hipLaunchKernelGGL((entmax_rows_bwd_kernel<T, AM_15>), dim3((unsigned)blocks), dim3(256), 0, s, y, dy, dx, rows, cols, cf);

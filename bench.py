@@ -10,6 +10,7 @@ Workloads (``--workload``):
   c3   adasplash_v2 causal MHA, B=4 H=16 N=4096 D=64 bf16, q pre-scaled by 1/sqrt(D)
   c5   adasplash_v1 non-causal alpha=1.333 niter=10, B=2 H=16 N=16384 D=64 bf16, q,k x3
   c2   entmax rows x[16384, 8192] = 4*N(0,1), bf16 and fp32, alpha in {1.5, 2}
+  c2_bwd  entmax rows backward on the same shape (reads y, writes dx, reads dy on the support only)
   c4_bwd, c3_bwd   dq, dk, dv of the c4 / c3 forward (2.5 x its dense-equivalent FLOPs per step)
 The default run also times the entmax rows workload (c2) and the c4 backward and reports them under ``extra``.
 
@@ -156,6 +157,42 @@ def bench_rows(steps, warmup, device, rows=16384, cols=8192):
     return out
 
 
+def bench_rows_backward(steps, warmup, device, rows=16384, cols=8192):
+    """Entmax rows backward on the forward's own outputs; buffers rotated as in ``bench_rows``.  The kernel
+    reads y, writes dx, and reads dy only where y is non-zero (a fraction of a percent of these rows), so the
+    algorithmic bytes are 2 * rows * cols * sizeof(dtype); counting dy in full would put the kernel above the
+    HBM peak."""
+    import adasplash_amd as A
+    from adasplash_amd import _lib
+
+    lib = _lib.load()
+    out = {}
+    g = torch.Generator().manual_seed(42)
+    base = 4.0 * torch.randn(rows, cols, generator=g)
+    for dt, dname in ((torch.bfloat16, "bf16"), (torch.float32, "f32")):
+        nbuf = 4
+        ys = [A.triton_entmax(base.roll(i, 0).to(dt).to(device), alpha=1.5) for i in range(nbuf)]
+        dys = [torch.randn(rows, cols, generator=g).to(dt).to(device) for _ in range(nbuf)]
+        dxs = [torch.empty_like(y) for y in ys]
+        nbytes = rows * cols * 2 * ys[0].element_size()
+        stream = _lib.current_stream(device)
+        state = {"i": 0}
+
+        def fn():
+            i = state["i"] % nbuf
+            st = lib.adsp_entmax_rows_bwd(ys[i].data_ptr(), dys[i].data_ptr(), dxs[i].data_ptr(), rows, cols,
+                                          _lib.dtype_code(ys[i]), 1.5, stream)
+            assert st == 0
+            state["i"] += 1
+
+        ms, _ = _events_ms(fn, max(steps, 20), max(warmup, 5))
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out[f"{dname}_alpha1.5"] = {"ms": ms, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS, "bytes": nbytes}
+        del ys, dys, dxs
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline():
     """Dense exact-entmax attention (the oracle) on the host cores, fp32 torch ops, on a bounded slice
     of the headline workload: B=1, Hq=4, Hkv=1, N=4096, D=128, causal, alpha=1.5."""
@@ -188,7 +225,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd", "c2_bwd"])
     ap.add_argument("--no-extra", action="store_true", help="skip the entmax-rows and CPU-baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -213,7 +250,16 @@ def main():
                      "config": {"workload": "copy: torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)"}})
         print(json.dumps(line))
         return
-    if args.workload == "c2":
+    if args.workload == "c2_bwd":
+        rows = bench_rows_backward(args.steps, args.warmup, device)
+        best = rows["f32_alpha1.5"]
+        line.update({"value": best["GBps"], "unit": "GB/s", "ms_per_step": best["ms"], "dtype": "f32",
+                     "config": {"workload": "c2_bwd: entmax rows backward [16384, 8192] fp32 alpha=1.5"},
+                     "roofline": {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": best["frac_hbm_peak"], "traffic": MEASURED_HBM_TRAFFIC_BYTES.get("c2_bwd_f32"),
+                                  "kernel": "entmax_rows_bwd_reg_kernel", "bytes_per_launch": best["bytes"]},
+                     "extra": {"entmax_rows_backward": rows}})
+    elif args.workload == "c2":
         rows = bench_rows(args.steps, args.warmup, device)
         best = rows["f32_alpha1.5"]
         line.update({"value": best["GBps"], "unit": "GB/s", "ms_per_step": best["ms"], "dtype": "f32",

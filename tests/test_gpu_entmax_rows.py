@@ -136,3 +136,46 @@ def test_backward_matches_finite_differences_of_the_oracle(alpha):
         w = torch.randn_like(x)
         fd = ((exact.entmax_rows(x + eps * w, alpha) - exact.entmax_rows(x - eps * w, alpha)) / (2 * eps) * dy).sum()
         assert abs((dx.double().cpu() * w).sum().item() - fd.item()) < 2e-3 * (1 + abs(fd.item()))
+
+
+def _rows_backward_reference(y, dy, alpha):
+    """dx = u * (dy - sum(u dy) / sum(u)), u = y^(2 - alpha) on the support (adasplash/triton_entmax_v2.py:541-617),
+    in fp64 torch ops on the kernel's own y."""
+    y64, g64 = y.double().cpu(), dy.double().cpu()
+    # generic alpha: the power is taken of max(y, 1e-6), the reference's clamp (triton_entmax_v2.py:35-39)
+    floor = 1e-300 if alpha in (1.5, 2.0) else 1e-6
+    u = torch.where(y64 > 0, y64.clamp_min(floor) ** (2.0 - alpha), torch.zeros_like(y64))
+    q = (u * g64).sum(-1, keepdim=True) / u.sum(-1, keepdim=True)
+    return u * (g64 - q)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("alpha", ALPHAS)
+@pytest.mark.parametrize("shape", [(64, 8192), (37, 4096), (5, 1000), (9, 24), (3, 16384), (2, 40000)])
+def test_backward_kernels_match_the_closed_form(shape, alpha, dtype):
+    """Every dispatch of the backward (a wave per row, a block per row, streaming for ragged or very long rows)
+    against the closed form; tolerance = the output type's rounding (fp32 1e-5, or 1e-4 where the power goes
+    through the hardware exp2 / log2; 16-bit 1e-2 of the largest |dx|)."""
+    g = torch.Generator().manual_seed(42)
+    x = (4 * torch.randn(*shape, generator=g)).to(dtype).to(DEV)
+    dy = torch.randn(*shape, generator=g).to(dtype).to(DEV)
+    xg = x.clone().requires_grad_(True)
+    y = A.triton_entmax(xg, alpha=alpha)
+    (dx,) = torch.autograd.grad(y, xg, dy)
+    want = _rows_backward_reference(y.detach(), dy, alpha)
+    tol = (1e-5 if alpha in (1.5, 2.0) else 1e-4) if dtype == torch.float32 else 1e-2  # generic alpha: exp2/log2 units
+    scale = max(1.0, want.abs().max().item())
+    assert (dx.double().cpu() - want).abs().max().item() < tol * scale
+    # entries outside the support get exactly zero
+    assert (dx[y == 0] == 0).all()
+
+
+def test_backward_of_an_all_zero_row_is_zero():
+    y = torch.zeros(4, 512, device=DEV)
+    dy = torch.randn(4, 512, device=DEV)
+    dx = torch.full_like(y, float("nan"))
+    from adasplash_amd import _lib
+    st = _lib.load().adsp_entmax_rows_bwd(y.data_ptr(), dy.data_ptr(), dx.data_ptr(), 4, 512, _lib.dtype_code(y), 1.5,
+                                          _lib.current_stream(y.device))
+    assert st == 0
+    assert (dx == 0).all()
