@@ -240,7 +240,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(rows_min_wa
   for (int c = 0; c < NCHUNK; ++c) {
     long long vi = (long long)c * TPR + t_in_row;
     r.valid[c] = vi < nvec;
-    if (r.valid[c]) r.raw[c] = __builtin_nontemporal_load(xrow + vi);
+    // a lane past the row end re-reads the row's last chunk and ignores it: no branch between the loads
+    r.raw[c] = __builtin_nontemporal_load(xrow + (r.valid[c] ? vi : nvec - 1));
   }
   if (t_in_row == 0) cand_n[r_in_blk] = 0;
 
