@@ -167,6 +167,43 @@ def dense_entmax_attention(q, k, v, alpha=1.5, is_causal=False, varlen=None, dty
     return out
 
 
+def dense_entmax_attention_general(q, k, v, alpha=1.5, is_causal=False, varlen=None, padding="right",
+                                   alibi_slopes=None, dtype=torch.float64):
+    """The dense example path with all its options (``examples/attention.py:8-31,34-91``), exact entmax, fp64.
+
+    ALiBi adds ``slope_h * (j - i)`` to the score of query ``i`` and key ``j`` (``j - (k_len - 1)`` for a single
+    query row); ``padding="left"`` keeps the *last* ``varlen[b]`` positions; a causal mask with
+    ``q_len != k_len`` is aligned to the bottom right; padded query rows (only defined when
+    ``q_len == k_len``) are zero.  Written as explicit loops over batch and head so that it shares no tensor
+    expression with the implementation under test.
+    """
+    B, H, Nq, D = q.shape
+    Nk = k.shape[2]
+    out = torch.zeros(B, H, Nq, v.shape[3], dtype=dtype)
+    for b in range(B):
+        if varlen is None:
+            keys = list(range(Nk))
+        else:
+            L = int(varlen[b])
+            keys = list(range(L)) if padding == "right" else list(range(Nk - L, Nk))
+        keyset = set(keys)
+        for h in range(H):
+            for i in range(Nq):
+                if varlen is not None and Nq == Nk and i not in keyset:
+                    continue  # padded query row: zero
+                pos_i = i + (Nk - Nq)  # position of the query among the keys (bottom-right alignment)
+                cols = [j for j in keys if (not is_causal) or j <= pos_i]
+                if not cols:
+                    continue
+                s = (k[b, h, cols].to(dtype) @ q[b, h, i].to(dtype)) / math.sqrt(D)
+                if alibi_slopes is not None:
+                    ref_i = (Nk - 1) if (Nq == 1 and Nk > 1) else i
+                    s = s + float(alibi_slopes[h]) * (torch.tensor(cols, dtype=dtype) - ref_i)
+                p = entmax_rows(s[None, :], alpha, dtype=dtype)[0]
+                out[b, h, i] = p @ v[b, h, cols].to(dtype)
+    return out
+
+
 def dense_entmax_attention_grads(q, k, v, dout, alpha=1.5, is_causal=False, varlen=None, dtype=torch.float64):
     """Gradients (dq, dk, dv) of ``dense_entmax_attention`` for the upstream gradient ``dout``.
 

@@ -211,3 +211,67 @@ def test_closed_form_gradients_match_finite_differences(alpha, causal, shape, va
             flat[i] = old
             num[i] = (fp - fm) / (2 * eps)
         assert (num.view_as(gr) - gr).abs().max() < 1e-7
+
+
+# ---- the dense example path with ALiBi, left padding and q_len != k_len (examples/attention.py:8-91) ----------
+
+def _rand_qkv(B, H, Nq, Nk, D, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(B, H, Nq, D, generator=g, dtype=torch.float64), torch.randn(B, H, Nk, D, generator=g, dtype=torch.float64),
+            torch.randn(B, H, Nk, D, generator=g, dtype=torch.float64))
+
+
+def test_general_dense_path_reduces_to_the_plain_oracle():
+    q, k, v = _rand_qkv(2, 2, 12, 12, 8)
+    vl = torch.tensor([7, 12])
+    for alpha in (1.5, 2.0, 1.333):
+        for causal in (False, True):
+            a = exact.dense_entmax_attention(q, k, v, alpha, causal, varlen=vl)
+            b = exact.dense_entmax_attention_general(q, k, v, alpha, causal, varlen=vl)
+            assert (a - b).abs().max().item() < 1e-9
+
+
+def test_alibi_sign_and_row_shift_invariance():
+    """A large positive slope must pull a causal row onto its most recent key (out_i -> v_i): a bias of the wrong
+    sign, or taken over queries instead of keys, sends it to the first key or changes nothing.  And the bias of a
+    row, slope * (j - i), differs from slope * j by a per-row constant, which entmax ignores."""
+    q, k, v = _rand_qkv(1, 2, 10, 10, 4, seed=1)
+    out = exact.dense_entmax_attention_general(q, k, v, 1.5, True, alibi_slopes=torch.tensor([60.0, 80.0]))
+    assert (out - v).abs().max().item() < 1e-9
+    slopes = torch.tensor([0.3, 0.05])
+    got = exact.dense_entmax_attention_general(q, k, v, 1.5, True, alibi_slopes=slopes)
+    # same thing by hand: fold slope * j into the scores through an extra (q, k) feature pair
+    D = q.shape[-1]
+    j = torch.arange(10, dtype=torch.float64)
+    q2 = torch.cat([q, torch.ones(1, 2, 10, 1, dtype=torch.float64)], -1) * math.sqrt((D + 1) / D)
+    k2 = torch.cat([k, (slopes[:, None] * j[None, :])[None, :, :, None] * math.sqrt(D)], -1)
+    want = exact.dense_entmax_attention(q2, k2, v, 1.5, True)
+    assert (got - want).abs().max().item() < 1e-9
+    # without a causal mask the bias is not a row shift of anything simpler, but slope 0 must be a no-op
+    a = exact.dense_entmax_attention_general(q, k, v, 2.0, False, alibi_slopes=torch.zeros(2))
+    assert (a - exact.dense_entmax_attention(q, k, v, 2.0, False)).abs().max().item() < 1e-12
+
+
+def test_left_padding_is_the_unpadded_problem_at_the_end():
+    q, k, v = _rand_qkv(2, 2, 9, 9, 4, seed=2)
+    vl = torch.tensor([5, 9])
+    for causal in (False, True):
+        out = exact.dense_entmax_attention_general(q, k, v, 1.5, causal, varlen=vl, padding="left")
+        assert (out[0, :, :4] == 0).all()
+        tail = exact.dense_entmax_attention(q[:1, :, 4:], k[:1, :, 4:], v[:1, :, 4:], 1.5, causal)
+        assert (out[:1, :, 4:] - tail).abs().max().item() < 1e-9
+        full = exact.dense_entmax_attention(q[1:], k[1:], v[1:], 1.5, causal)
+        assert (out[1:] - full).abs().max().item() < 1e-9
+
+
+def test_bottom_right_causal_mask_and_single_query_alibi():
+    """q_len < k_len: the queries are the last q_len positions, so the result is the tail of the square problem;
+    a single query row takes the ALiBi bias of the last position."""
+    q, k, v = _rand_qkv(1, 2, 11, 11, 4, seed=3)
+    slopes = torch.tensor([0.2, 0.7])
+    square = exact.dense_entmax_attention_general(q, k, v, 1.5, True)
+    tail = exact.dense_entmax_attention_general(q[:, :, -3:], k, v, 1.5, True)
+    assert (square[:, :, -3:] - tail).abs().max().item() < 1e-9
+    sq_alibi = exact.dense_entmax_attention_general(q, k, v, 1.5, True, alibi_slopes=slopes)
+    one = exact.dense_entmax_attention_general(q[:, :, -1:], k, v, 1.5, True, alibi_slopes=slopes)
+    assert (sq_alibi[:, :, -1:] - one).abs().max().item() < 1e-9

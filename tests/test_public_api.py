@@ -170,3 +170,18 @@ def test_argument_errors_come_back_as_status_codes():
     assert lib.adsp_attn_v2_fwd(16, 16, 16, 16, None, None, None, 0, 1, 1, 1, 64, 64, 1, 1, None, 0, None) == 6
     assert lib.adsp_attn_v1_fwd(16, 16, 16, 16, None, None, None, 0, 1, 1, 64, 64, 0, 2.5, 0, 1, None, 0, None,
                                 None) == 5
+
+
+def test_dense_example_names_and_signatures():
+    """``examples/attention.py:34-44,94``: the dense path and the dispatcher alias keep their argument lists."""
+    import inspect
+
+    from adasplash_amd import dense
+
+    sig = inspect.signature(dense.slow_entmax_attention)
+    assert list(sig.parameters) == ["q", "k", "v", "alpha", "varlen", "is_causal", "padding", "niter", "alibi_slopes"]
+    assert [sig.parameters[n].default for n in ("alpha", "varlen", "is_causal", "padding", "niter", "alibi_slopes")] == \
+        [1.5, None, False, "right", 2, None]
+    sig = inspect.signature(dense.flash_entmax_attention)
+    assert list(sig.parameters) == ["q", "k", "v", "alpha", "varlen", "is_causal", "niter"]
+    assert sig.parameters["is_causal"].default is True
