@@ -48,15 +48,31 @@ template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t w) { retu
 template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t w) { return f16_bits_to_float(w >> 16); }
 
 // ---- wave64 butterflies ---------------------------------------------------------------------------
+// Wave-wide reductions on the DPP network (row shifts, then the two row broadcasts of this ISA family); the
+// result is read from lane 63 into a scalar register, so every lane gets it.  All 64 lanes must be active.
+// Six VALU instructions, against six LDS-crossbar round trips for the same reduction written with shuffles.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), CTRL,
+                                                               ROW_MASK, 0xf, false));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fmaxf(v, dpp_move<0x111, 0xf>(-INFINITY, v));  // row_shr:1
+  v = fmaxf(v, dpp_move<0x112, 0xf>(-INFINITY, v));  // row_shr:2
+  v = fmaxf(v, dpp_move<0x114, 0xf>(-INFINITY, v));  // row_shr:4
+  v = fmaxf(v, dpp_move<0x118, 0xf>(-INFINITY, v));  // row_shr:8: lane 15 of a row holds the row's result
+  v = fmaxf(v, dpp_move<0x142, 0xa>(-INFINITY, v));  // row_bcast:15 into rows 1 and 3
+  v = fmaxf(v, dpp_move<0x143, 0xc>(-INFINITY, v));  // row_bcast:31 into rows 2 and 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  v += dpp_move<0x111, 0xf>(0.f, v);
+  v += dpp_move<0x112, 0xf>(0.f, v);
+  v += dpp_move<0x114, 0xf>(0.f, v);
+  v += dpp_move<0x118, 0xf>(0.f, v);
+  v += dpp_move<0x142, 0xa>(0.f, v);
+  v += dpp_move<0x143, 0xc>(0.f, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
