@@ -17,6 +17,7 @@
 // The 16-bit path takes the transposed operands (K^T, dO^T, Q^T) from tile-wise transposed copies in the
 // layout of vt_layout_kernel, so that P / dX go from the accumulators straight into the next MFMA.
 #pragma once
+#include <type_traits>
 #include "attn_kernel.h"
 #include "attn_bwd_params.h"
 
@@ -281,6 +282,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   const bool live = qi < L;
   const float tau = live ? p.taus[q_base + qi] : INFINITY;
   const int lim = p.causal ? (qi < L - 1 ? qi : L - 1) : L - 1;  // last valid key of the lane's row
+  const int lim_all = p.causal ? (wave_row0 < L - 1 ? wave_row0 : L - 1) : L - 1;  // smallest `lim` of the wave (wave-uniform)
   const int row_hi = (m0 + kBwdRows < L ? m0 + kBwdRows : L);
   const int nt = p.causal ? (row_hi + kBN - 1) / kBN : (L + kBN - 1) / kBN;
   const int32_t* mrow = p.bmask ? p.bmask + ((size_t)bh * p.n_mblk + mblk) * p.mask_words : nullptr;
@@ -340,16 +342,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
       }
     }
   };
-  // r = z - tau for the 16 keys of block kb (-inf where the row may not look), and dP.
-  auto block_terms = [&](int kt, int kb, const unsigned char* ka, const unsigned char* va, float (&r)[16], f32x16& dp) {
+  // r = z - tau for the 16 keys of block kb (-inf where the row may not look), and dP.  A block that every row of
+  // the wave sees in full (below the causal diagonal, inside the sequence) is "plain": no per-score predicate,
+  // one fma per score instead of a compare and two selects more.  The choice is a template argument so that each
+  // kind of block is one piece of straight-line code, products included.
+  // (only where the second code path fits the register budget: at D = 128 it costs spills and more than it saves)
+  constexpr bool kPlainBlocks = k16 && D <= 64;
+  auto block_is_plain = [&](int kt, int kb) { return kPlainBlocks && kt * kBN + kb * 32 + 31 <= lim_all; };
+  auto block_terms = [&](auto plain_c, int kt, int kb, const unsigned char* ka, const unsigned char* va, float (&r)[16],
+                         f32x16& dp) {
     f32x16 s = BT::dot_block(ka, kb, qf, lq, lh);
     dp = BT::dot_block(va, kb, dof, lq, lh);
-    const int jb = kt * kBN + kb * 32 + 4 * lh;
+    if constexpr (decltype(plain_c)::value) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const bool ok = jb + 8 * (i >> 2) + (i & 3) <= lim;
-      r[i] = ok ? fmaf(s[i], p.qscale, -tau) : -INFINITY;
-      dp[i] = ok ? dp[i] : 0.f;  // keys past the end may hold anything
+      for (int i = 0; i < 16; ++i) r[i] = fmaf(s[i], p.qscale, -tau);
+    } else {
+      const int jb = kt * kBN + kb * 32 + 4 * lh;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bool ok = jb + 8 * (i >> 2) + (i & 3) <= lim;
+        r[i] = ok ? fmaf(s[i], p.qscale, -tau) : -INFINITY;
+        dp[i] = ok ? dp[i] : 0.f;  // keys past the end may hold anything
+      }
     }
   };
 
@@ -360,16 +374,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
-      float r[16];
-      f32x16 dp;
-      block_terms(kt, kb, ka, va, r, dp);
+      auto block = [&](auto plain_c) {
+        float r[16];
+        f32x16 dp;
+        block_terms(plain_c, kt, kb, ka, va, r, dp);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float pr, u;
-        bwd_prob<AM>(r[i], p.c0, pr, u);
-        zsum += pr;
-        usum += u;
-        udp = fmaf(u, dp[i], udp);
+        for (int i = 0; i < 16; ++i) {
+          float pr, u;
+          bwd_prob<AM>(r[i], p.c0, pr, u);
+          zsum += pr;
+          usum += u;
+          udp = fmaf(u, dp[i], udp);
+        }
+      };
+      if constexpr (!kPlainBlocks) {
+        block(std::false_type{});
+      } else if (block_is_plain(kt, kb)) {
+        asm volatile("; plain block" ::: "memory");
+        block(std::true_type{});
+      } else {
+        asm volatile("; masked block" ::: "memory");
+        block(std::false_type{});
       }
     }
   });
@@ -393,17 +418,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
-      float r[16];
-      f32x16 dp;
-      block_terms(kt, kb, ka, va, r, dp);
-      float dx[16];
+      auto block = [&](auto plain_c) {
+        float r[16];
+        f32x16 dp;
+        block_terms(plain_c, kt, kb, ka, va, r, dp);
+        float dx[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float pr, u;
-        bwd_prob<AM>(r[i], p.c0, pr, u);
-        dx[i] = u * (dp[i] - delta);
+        for (int i = 0; i < 16; ++i) {
+          float pr, u;
+          bwd_prob<AM>(r[i], p.c0, pr, u);
+          dx[i] = u * (dp[i] - delta);
+        }
+        BT::acc_block(acc, k16 ? kta : ka, kb, dx, lq, lh, L - kt * kBN);
+      };
+      if constexpr (!kPlainBlocks) {
+        block(std::false_type{});
+      } else if (block_is_plain(kt, kb)) {
+        asm volatile("; plain block" ::: "memory");
+        block(std::true_type{});
+      } else {
+        asm volatile("; masked block" ::: "memory");
+        block(std::false_type{});
       }
-      BT::acc_block(acc, k16 ? kta : ka, kb, dx, lq, lh, L - kt * kBN);
     }
   });
 
@@ -552,17 +588,76 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
     }
   };
   // r = z - tau_i for the 16 queries of block qb against the lane's key (-inf where query i may not see it)
-  auto block_r = [&](int qt, int qb, const unsigned char* qa, const float (*sc)[kBN], float (&r)[16]) {
+  // Returns true for a plain block: every key of the wave is seen by every query of the block (all inside the
+  // sequence, the block below the causal diagonal).  Such a block needs no per-score predicate, and the selects
+  // that keep 0 x (anything in a padding row) out of the gradients can go too.
+  auto block_r = [&](int qt, int qb, const unsigned char* qa, const float (*sc)[kBN], float (&r)[16]) -> bool {
     f32x16 s = BT::dot_block(qa, qb, kf, lq, lh);
+    const int q_first = qt * kBN + qb * 32;
+    const bool plain = wave_key0 + 31 < L && q_first + 31 < L && (!p.causal || wave_key0 + 31 <= q_first);
+    if (plain) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 tq = *reinterpret_cast<const f32x4*>(&sc[0][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[4 * g + e] = fmaf(s[4 * g + e], p.qscale, -tq[e]);
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 tq = *reinterpret_cast<const f32x4*>(&sc[0][qb * 32 + 8 * g + 4 * lh]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * g + e;
+          const int qrow = q_first + 8 * g + 4 * lh + e;
+          const bool ok = key_live && qrow < L && (!p.causal || kj <= qrow);
+          r[i] = ok ? fmaf(s[i], p.qscale, -tq[e]) : -INFINITY;
+        }
+      }
+    }
+    return plain;
+  };
+  // MFMA operands of the two gradient products from r: p / sum p for dV, u (dP - delta) for dK.  Outside plain
+  // blocks a zero weight is selected, not multiplied: its partner may sit in a padding row and hold anything.
+  auto weights_p = [&](bool plain, int qb, const float (&r)[16], const float (*sc)[kBN], float (&w)[16]) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const f32x4 tq = *reinterpret_cast<const f32x4*>(&sc[0][qb * 32 + 8 * g + 4 * lh]);
+      const f32x4 zi = *reinterpret_cast<const f32x4*>(&sc[1][qb * 32 + 8 * g + 4 * lh]);
+      if (plain) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int i = 4 * g + e;
-        const int qrow = qt * kBN + qb * 32 + 8 * g + 4 * lh + e;
-        const bool ok = key_live && qrow < L && (!p.causal || kj <= qrow);
-        r[i] = ok ? fmaf(s[i], p.qscale, -tq[e]) : -INFINITY;
+        for (int e = 0; e < 4; ++e) {
+          float pr, u;
+          bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+          w[4 * g + e] = pr * zi[e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float pr, u;
+          bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+          w[4 * g + e] = pr > 0.f ? pr * zi[e] : 0.f;
+        }
+      }
+    }
+  };
+  auto weights_x = [&](bool plain, int qb, const float (&r)[16], const f32x16& dp, const float (*sc)[kBN], float (&w)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 di = *reinterpret_cast<const f32x4*>(&sc[2][qb * 32 + 8 * g + 4 * lh]);
+      if (plain) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float pr, u;
+          bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+          w[4 * g + e] = u * (dp[4 * g + e] - di[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float pr, u;
+          bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
+          w[4 * g + e] = u > 0.f ? u * (dp[4 * g + e] - di[e]) : 0.f;
+        }
       }
     }
   };
@@ -591,31 +686,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
                   for (int qb = 0; qb < 2; ++qb) {
                     if (!block_visible(qt, qb)) continue;
                     float r[16], w[16];
-                    block_r(qt, qb, qa, sc, r);
+                    const bool plain = block_r(qt, qb, qa, sc, r);
                     // dV first: p / sum p
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                      const f32x4 zi = *reinterpret_cast<const f32x4*>(&sc[1][qb * 32 + 8 * g + 4 * lh]);
-#pragma unroll
-                      for (int e = 0; e < 4; ++e) {
-                        float pr, u;
-                        bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
-                        w[4 * g + e] = pr > 0.f ? pr * zi[e] : 0.f;
-                      }
-                    }
+                    weights_p(plain, qb, r, sc, w);
                     BT::acc_block(acc, dota, qb, w, lq, lh, L - qt * kBN);
                     // then dK: u (dP - delta)
                     f32x16 dp = BT::dot_block(doa, qb, vf, lq, lh);
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                      const f32x4 di = *reinterpret_cast<const f32x4*>(&sc[2][qb * 32 + 8 * g + 4 * lh]);
-#pragma unroll
-                      for (int e = 0; e < 4; ++e) {
-                        float pr, u;
-                        bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
-                        w[4 * g + e] = u > 0.f ? u * (dp[4 * g + e] - di[e]) : 0.f;
-                      }
-                    }
+                    weights_x(plain, qb, r, dp, sc, w);
                     BT::acc_block(acc_k, qta, qb, w, lq, lh, L - qt * kBN);
                   }
                 });
@@ -640,17 +717,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
                 for (int qb = 0; qb < 2; ++qb) {
                   if (!block_visible(qt, qb)) continue;
                   float r[16], w[16];
-                  block_r(qt, qb, qa, sc, r);
-#pragma unroll
-                  for (int g = 0; g < 4; ++g) {
-                    const f32x4 zi = *reinterpret_cast<const f32x4*>(&sc[1][qb * 32 + 8 * g + 4 * lh]);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                      float pr, u;
-                      bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
-                      w[4 * g + e] = pr > 0.f ? pr * zi[e] : 0.f;
-                    }
-                  }
+                  const bool plain = block_r(qt, qb, qa, sc, r);
+                  weights_p(plain, qb, r, sc, w);
                   BT::acc_block(acc, k16 ? ta : doa, qb, w, lq, lh, L - qt * kBN);
                 }
               });
@@ -671,18 +739,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
                 for (int qb = 0; qb < 2; ++qb) {
                   if (!block_visible(qt, qb)) continue;
                   float r[16], w[16];
-                  block_r(qt, qb, qa, sc, r);
+                  const bool plain = block_r(qt, qb, qa, sc, r);
                   f32x16 dp = BT::dot_block(doa, qb, vf, lq, lh);
-#pragma unroll
-                  for (int g = 0; g < 4; ++g) {
-                    const f32x4 di = *reinterpret_cast<const f32x4*>(&sc[2][qb * 32 + 8 * g + 4 * lh]);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                      float pr, u;
-                      bwd_prob<AM>(r[4 * g + e], p.c0, pr, u);
-                      w[4 * g + e] = u > 0.f ? u * (dp[4 * g + e] - di[e]) : 0.f;
-                    }
-                  }
+                  weights_x(plain, qb, r, dp, sc, w);
                   BT::acc_block(acc, k16 ? ta : qa, qb, w, lq, lh, L - qt * kBN);
                 }
               });
