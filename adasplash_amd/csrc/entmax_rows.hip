@@ -455,7 +455,7 @@ template <typename T, int AM, int NCHUNK, int TPR> static void launch_reg(const 
   hipLaunchKernelGGL((entmax_rows_reg_kernel<T, AM, NCHUNK, TPR>), dim3((unsigned)blocks), dim3(256), 0, s, p);
 }
 
-template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool aligned, int force_tpr, hipStream_t s) {
+template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool aligned, hipStream_t s) {
   constexpr int kVec = elem_traits<T>::kVec;
   const long long nvec = p.cols / kVec;
   const bool can_reg = aligned && (p.cols % kVec == 0) && p.rows < (1ll << 31);
@@ -465,9 +465,7 @@ template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool a
     // row beyond that, where more loads in flight per row pay more than the barriers cost (measured on
     // 2^27-element problems: bf16 4096 columns 74 % of HBM peak with a wave per row against 42 %, 8192
     // columns 66 % against 74-77 %).
-    int tpr = c64 <= 8 ? 64 : 256;
-    if (force_tpr == 64 && c64 <= 32) tpr = 64;
-    if (force_tpr == 256) tpr = 256;
+    const int tpr = c64 <= 8 ? 64 : 256;
     if (tpr == 64) {
       if (c64 <= 1) return launch_reg<T, AM, 1, 64>(p, s);
       if (c64 <= 2) return launch_reg<T, AM, 2, 64>(p, s);
@@ -488,10 +486,10 @@ template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool a
   hipLaunchKernelGGL((entmax_rows_stream_kernel<T, AM>), dim3((unsigned)blocks), dim3(256), 0, s, p);
 }
 
-template <typename T> static void launch_fwd_am(const RowsParams& p, int am, bool aligned, int force_tpr, hipStream_t s) {
-  if (am == AM_15) return launch_fwd<T, AM_15>(p, aligned, force_tpr, s);
-  if (am == AM_2) return launch_fwd<T, AM_2>(p, aligned, force_tpr, s);
-  return launch_fwd<T, AM_GEN>(p, aligned, force_tpr, s);
+template <typename T> static void launch_fwd_am(const RowsParams& p, int am, bool aligned, hipStream_t s) {
+  if (am == AM_15) return launch_fwd<T, AM_15>(p, aligned, s);
+  if (am == AM_2) return launch_fwd<T, AM_2>(p, aligned, s);
+  return launch_fwd<T, AM_GEN>(p, aligned, s);
 }
 
 template <typename T, int AM, int NCHUNK, int TPR>
@@ -538,10 +536,6 @@ static int alpha_mode(double alpha) { return alpha == 1.5 ? AM_15 : (alpha == 2.
 
 }  // namespace adsp
 
-// Tuning knob for experiments (0 = automatic, 64 = a wave per row, 256 = a block per row).
-static int g_rows_force_tpr = 0;
-extern "C" void adsp_debug_set_rows_threads_per_row(int tpr) { g_rows_force_tpr = tpr; }
-
 extern "C" int adsp_entmax_rows_fwd(const void* x, void* y, int64_t rows, int64_t cols, int dtype, double alpha,
                                     int n_iter, int use_histogram, int fast_math, void* stream) {
   using namespace adsp;
@@ -566,9 +560,9 @@ extern "C" int adsp_entmax_rows_fwd(const void* x, void* y, int64_t rows, int64_
   const bool aligned = (((uintptr_t)x | (uintptr_t)y) & 15) == 0;
   hipStream_t s = (hipStream_t)stream;
   (void)hipGetLastError();
-  if (dtype == ADSP_F32) launch_fwd_am<float>(p, am, aligned, g_rows_force_tpr, s);
-  else if (dtype == ADSP_BF16) launch_fwd_am<bf16_t>(p, am, aligned, g_rows_force_tpr, s);
-  else launch_fwd_am<f16_t>(p, am, aligned, g_rows_force_tpr, s);
+  if (dtype == ADSP_F32) launch_fwd_am<float>(p, am, aligned, s);
+  else if (dtype == ADSP_BF16) launch_fwd_am<bf16_t>(p, am, aligned, s);
+  else launch_fwd_am<f16_t>(p, am, aligned, s);
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
 }
 
