@@ -12,7 +12,7 @@ Workloads (``--workload``):
   c2   entmax rows x[16384, 8192] = 4*N(0,1), bf16 and fp32, alpha in {1.5, 2}
   c2_bwd  entmax rows backward on the same shape (reads y, writes dx, reads dy on the support only)
   c4_bwd, c3_bwd   dq, dk, dv of the c4 / c3 forward (2.5 x its dense-equivalent FLOPs per step)
-The default run also times the entmax rows workload (c2) and the c4 backward and reports them under ``extra``.
+The default run also times the entmax rows workloads (c2, c2_bwd) and the c4 backward and reports them under ``extra``.
 
 Dense-equivalent FLOPs of causal attention = 2 * Hq * D * sum_b L_b^2 (QK^T and PV, each halved by
 causality); non-causal = 4 * B * H * N^2 * D.  Rows bytes = rows * cols * (sizeof(in) + sizeof(out)).
@@ -284,6 +284,7 @@ def main():
             del res
             torch.cuda.empty_cache()
             line["extra"]["entmax_rows"] = bench_rows(args.steps, args.warmup, device)
+            line["extra"]["entmax_rows_backward"] = bench_rows_backward(args.steps, args.warmup, device)
             if args.workload == "c4":
                 b = bench_attention("c4", max(3, args.steps // 2), 1, device, backward=True)
                 line["extra"]["attention_backward"] = {k: b[k] for k in ("ms_per_step", "eff_tflops", "frac_mfma_peak",
