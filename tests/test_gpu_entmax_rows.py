@@ -179,3 +179,23 @@ def test_backward_of_an_all_zero_row_is_zero():
                                           _lib.current_stream(y.device))
     assert st == 0
     assert (dx == 0).all()
+
+
+def test_backward_with_unaligned_buffers_takes_the_streaming_path():
+    """y, dy and dx that are only 4-byte aligned cannot use 16-byte loads: same result through the fallback."""
+    from adasplash_amd import _lib
+    torch.manual_seed(5)
+    rows, cols = 6, 256
+    y_al = A.triton_entmax(4 * torch.randn(rows, cols, device=DEV), alpha=1.5)
+    dy_al = torch.randn(rows, cols, device=DEV)
+    bufs = [torch.empty(rows * cols + 1, device=DEV) for _ in range(3)]
+    y, dy, dx = (b[1:].view(rows, cols) for b in bufs)
+    y.copy_(y_al)
+    dy.copy_(dy_al)
+    assert all(t.data_ptr() % 16 != 0 for t in (y, dy, dx))
+    lib = _lib.load()
+    st = lib.adsp_entmax_rows_bwd(y.data_ptr(), dy.data_ptr(), dx.data_ptr(), rows, cols, _lib.dtype_code(y), 1.5,
+                                  _lib.current_stream(y.device))
+    assert st == 0
+    want = _rows_backward_reference(y_al, dy_al, 1.5)
+    assert (dx.double().cpu() - want).abs().max().item() < 1e-5
