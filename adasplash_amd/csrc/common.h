@@ -74,6 +74,22 @@ __device__ __forceinline__ float wave_sum(float v) {
   v += dpp_move<0x143, 0xc>(0.f, v);
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// The same within every aligned group of 16 lanes (a DPP row): xor-butterflies over the quad, then the two
+// mirrors; every lane of the group ends with the group's result.  Lanes of a group must be active together.
+__device__ __forceinline__ float group16_max(float v) {
+  v = fmaxf(v, dpp_move<0xb1, 0xf>(v, v));   // quad_perm [1, 0, 3, 2]
+  v = fmaxf(v, dpp_move<0x4e, 0xf>(v, v));   // quad_perm [2, 3, 0, 1]
+  v = fmaxf(v, dpp_move<0x141, 0xf>(v, v));  // row_half_mirror
+  v = fmaxf(v, dpp_move<0x140, 0xf>(v, v));  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float group16_sum(float v) {
+  v += dpp_move<0xb1, 0xf>(v, v);
+  v += dpp_move<0x4e, 0xf>(v, v);
+  v += dpp_move<0x141, 0xf>(v, v);
+  v += dpp_move<0x140, 0xf>(v, v);
+  return v;
+}
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -29,6 +29,7 @@ struct RowsParams {
 
 // ---- reductions across the TPR threads that share a row ---------------------------------------------
 template <int TPR> __device__ __forceinline__ float row_max(float v, float* sm) {
+  if constexpr (TPR == 16) return group16_max(v);
   v = wave_max(v);
   if constexpr (TPR > 64) {
     __syncthreads();
@@ -41,6 +42,11 @@ template <int TPR> __device__ __forceinline__ float row_max(float v, float* sm) 
   return v;
 }
 template <int TPR, int K> __device__ __forceinline__ void row_sum(float (&v)[K], float* sm) {
+  if constexpr (TPR == 16) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = group16_sum(v[k]);
+    return;
+  }
 #pragma unroll
   for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
   if constexpr (TPR > 64) {
@@ -198,10 +204,11 @@ template <int K> struct ListRow {
 #pragma unroll
     for (int i = 0; i < K; ++i) f(z[i]);
   }
-  __device__ __forceinline__ void load(const float* list, int n, int lane) {
+  // thread t of the `stride` threads that solve the list takes entries t, t + stride, ...
+  __device__ __forceinline__ void load(const float* list, int n, int t, int stride = 64) {
 #pragma unroll
     for (int i = 0; i < K; ++i) {
-      const int idx = i * 64 + lane;
+      const int idx = i * stride + t;
       z[i] = idx < n ? list[idx] : -INFINITY;
     }
   }
@@ -218,7 +225,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(rows_min_wa
   constexpr int kVec = elem_traits<T>::kVec;
   constexpr int kRowsPerBlock = 256 / TPR;
   __shared__ float sm[32];
-  __shared__ float cand[kRowsPerBlock][kCandCap];
+  // Short rows (16 threads each, four to a wave): the row's own 16 lanes solve its list.
+  constexpr int kCap = TPR == 16 ? (NCHUNK * TPR * kVec < 512 ? NCHUNK * TPR * kVec : 512) : kCandCap;
+  __shared__ float cand[kRowsPerBlock][kCap];
   __shared__ int cand_n[kRowsPerBlock];
   const int tid = threadIdx.x;
   const int t_in_row = tid % TPR, r_in_blk = tid / TPR, lane = tid & 63;
@@ -283,7 +292,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(rows_min_wa
         const float x = chunk_elem<T>(r.raw[c], e);
         if (x >= x_thr) {
           const int idx = atomicAdd(&cand_n[r_in_blk], 1);
-          if (idx < kCandCap) cand[r_in_blk][idx] = x * p.scale;
+          if (idx < kCap) cand[r_in_blk][idx] = x * p.scale;
         }
       }
     }
@@ -292,7 +301,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(rows_min_wa
   const int n_cand = cand_n[r_in_blk];
 
   float tau;
-  if (n_cand <= 64) {
+  if constexpr (TPR == 16) {
+    if (n_cand <= 16) {
+      ListRow<1> lr;
+      lr.load(cand[r_in_blk], n_cand, t_in_row, 16);
+      tau = solve_row<AM, 16>(lr, p, sm);
+    } else if (n_cand <= kCap) {
+      ListRow<kCap / 16> lr;
+      lr.load(cand[r_in_blk], n_cand, t_in_row, 16);
+      tau = solve_row<AM, 16>(lr, p, sm);
+    } else {
+      StreamRow<T, 16> sr{p.x, (size_t)row * p.cols, p.cols, p.scale, t_in_row};
+      tau = solve_row<AM, 16>(sr, p, sm);
+    }
+  } else if (n_cand <= 64) {
     // every wave of the row solves the same short list redundantly: wave-level reductions only.  The
     // usual case (a peaked row) has at most one candidate per lane.
     ListRow<1> lr;
@@ -465,6 +487,17 @@ template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool a
     // row beyond that, where more loads in flight per row pay more than the barriers cost (measured on
     // 2^27-element problems: bf16 4096 columns 74 % of HBM peak with a wave per row against 42 %, 8192
     // columns 66 % against 74-77 %).
+    const long long c16 = (nvec + 15) / 16;
+#ifndef ADSP_ROWS_C16_MAX
+#define ADSP_ROWS_C16_MAX 8
+#endif
+    // Short rows: 16 threads per row, four rows to a wave, so that the per-row solve is shared out.
+    if (c16 <= ADSP_ROWS_C16_MAX) {
+      if (c16 <= 1) return launch_reg<T, AM, 1, 16>(p, s);
+      if (c16 <= 2) return launch_reg<T, AM, 2, 16>(p, s);
+      if (c16 <= 4) return launch_reg<T, AM, 4, 16>(p, s);
+      if (c16 <= 8) return launch_reg<T, AM, 8, 16>(p, s);
+    }
     const int tpr = c64 <= 8 ? 64 : 256;
     if (tpr == 64) {
       if (c64 <= 1) return launch_reg<T, AM, 1, 64>(p, s);
@@ -508,6 +541,11 @@ static bool launch_bwd_fast(const void* y, const void* dy, void* dx, long long r
   if (!aligned || cols % kVec != 0 || rows >= (1ll << 31)) return false;
   const long long nvec = cols / kVec;
   const long long c64 = (nvec + 63) / 64, c256 = (nvec + 255) / 256;
+  const long long c16 = (nvec + 15) / 16;  // short rows: 16 threads per row, four rows to a wave
+  if (c16 <= 1) return launch_bwd_reg<T, AM, 1, 16>(y, dy, dx, rows, cols, cf, s), true;
+  if (c16 <= 2) return launch_bwd_reg<T, AM, 2, 16>(y, dy, dx, rows, cols, cf, s), true;
+  if (c16 <= 4) return launch_bwd_reg<T, AM, 4, 16>(y, dy, dx, rows, cols, cf, s), true;
+  if (c16 <= 8) return launch_bwd_reg<T, AM, 8, 16>(y, dy, dx, rows, cols, cf, s), true;
   if (c64 <= 1) return launch_bwd_reg<T, AM, 1, 64>(y, dy, dx, rows, cols, cf, s), true;
   if (c64 <= 2) return launch_bwd_reg<T, AM, 2, 64>(y, dy, dx, rows, cols, cf, s), true;
   if (c64 <= 4) return launch_bwd_reg<T, AM, 4, 64>(y, dy, dx, rows, cols, cf, s), true;

@@ -199,3 +199,19 @@ def test_backward_with_unaligned_buffers_takes_the_streaming_path():
     assert st == 0
     want = _rows_backward_reference(y_al, dy_al, 1.5)
     assert (dx.double().cpu() - want).abs().max().item() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("alpha", ALPHAS)
+@pytest.mark.parametrize("cols", [8, 16, 24, 64, 128, 136, 256, 512, 520, 1024, 1032, 2048, 4096, 4104])
+def test_forward_across_the_dispatch_boundaries(cols, alpha, dtype):
+    """Row lengths on both sides of every switch between the kernel variants (16 threads per row with 1-8 chunks
+    per lane, a wave per row, four waves per row) and row counts that leave the last wave / block partly empty."""
+    g = torch.Generator().manual_seed(cols)
+    x = (3 * torch.randn(37, cols, generator=g)).to(dtype)
+    y = A.triton_entmax(x.to(DEV), alpha=alpha)
+    assert max_err(y, exact.entmax_rows(x, alpha)) < tol_for(dtype, alpha)
+    # a flat row has full support: every candidate list overflows its fast path
+    flat = torch.zeros(5, cols).to(dtype)
+    y = A.triton_entmax(flat.to(DEV), alpha=alpha)
+    assert (y.float().cpu() - 1.0 / cols).abs().max().item() < (1e-6 if dtype == torch.float32 else 2e-3 / cols + 1e-4)
