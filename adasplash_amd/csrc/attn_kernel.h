@@ -15,12 +15,13 @@
 // Passes over the K tiles of a row block (every pass recomputes S^T with MFMA; scores never leave
 // registers).  s = q.k is kept in raw units and the (alpha-1)/sqrt(D) scale is applied to per-row
 // scalars only, so the MFMA operands are the caller's q and k bit for bit:
-//   A  row max m                                          -> tau in [m - 1, m - n^(1-alpha)]
-//   B  (alpha = 1.5 / 2) 8-bin histogram of z - (m - 1)   -> bracket [lo, lo + 1/8]; tile mask {z > m-1}
-//   C  x niter: sums of u^c0, u^(c0-1), u^(c0-2)          -> Halley / Newton / bisection step; the last
-//                                                           one refines the tile mask to {z > lo}
+//   A+B (alpha = 1.5 / 2) row max m and, in the same walk, a histogram of z on an absolute grid of bins of width
+//      1/8 under the running maximum -> bracket [lo, lo + 1/8] of tau; tile mask {z within 1 of the running max}
+//   A  (other alpha) row max m                            -> tau in [m - 1, m - n^(1-alpha)]
+//   C  x niter: sums of u^c0, u^(c0-1), u^(c0-2)          -> Halley / Newton / bisection step; every one
+//                                                           refines the tile mask to {z > lower bound}
 //   D  p = [z - tau]_+^c0, out += P V over masked tiles, divided by sum p at the end.
-// The accumulator of the S^T MFMA is initialised with -tau (resp. -(m-1)), so z - tau costs no VALU op.
+// In walks C and D the accumulator of the S^T MFMA is initialised with -tau, so z - tau costs no VALU op.
 //
 // The 16-bit path consumes V through a tile-wise key-major copy (vt_layout_kernel) so that the PV product
 // out^T = V^T P^T can take P^T straight from the S^T accumulators without an LDS round trip.
