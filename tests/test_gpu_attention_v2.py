@@ -178,3 +178,18 @@ def test_v_of_ones_returns_ones_and_linearity_in_v():
     assert (ones.cpu() - 1).abs().max().item() < 1e-5
     a, b, c = run_v2(q, k, v1), run_v2(q, k, v2), run_v2(q, k, v1 + v2)
     assert (a + b - c).abs().max().item() < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_all_equal_scores_on_a_long_sequence_give_running_means(dtype):
+    """q = 0: every score of a row is equal, so every key lands in the top histogram bin and the row's
+    probabilities are uniform; out_i is the mean of v_0..v_i.  With N = 32768 a lane counts 16384 entries in one
+    bin, which exercises the upper bit planes of the histogram counters (carries out of the per-tile adder tree)."""
+    torch.manual_seed(0)
+    n = 32768
+    q = torch.zeros(1, 1, n, 64).to(dtype)
+    k = torch.randn(1, 1, n, 64).to(dtype)
+    v = torch.randn(1, 1, n, 64).to(dtype)
+    out = run_v2(q, k, v, niter=1).double().cpu()
+    want = v.double().cumsum(2) / torch.arange(1, n + 1, dtype=torch.float64).view(1, 1, n, 1)
+    assert (out - want).abs().max().item() < (1e-4 if dtype == torch.float32 else 1e-2)
