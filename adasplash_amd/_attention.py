@@ -54,8 +54,8 @@ def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
     """Enqueue the dQ and dK/dV kernels on the current stream; returns ``(dq, dk, dv)``.
 
     ``taus`` / ``bmask`` are the thresholds and the tile mask the forward produced.  Rows of ``dout`` past a
-    sequence's valid length are ignored (zeroed here, as the reference's masked loads do,
-    adasplash/adasplash_v2.py:1030-1033).
+    sequence's valid length are never used, whatever they hold (the kernels mask them as the reference's
+    loads do, adasplash/adasplash_v2.py:1030-1033).
     """
     _lib.require_device(q, k, v, dout, varlen)
     lib = _lib.load()
@@ -63,9 +63,6 @@ def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
     Hkv = k.shape[1]
     dt = _lib.dtype_code(q)
     dout = dout.to(q.dtype).contiguous()
-    if varlen is not None:
-        valid = torch.arange(N, device=q.device)[None, :] < varlen.to(torch.long)[:, None]
-        dout = torch.where(valid[:, None, :, None], dout, torch.zeros((), device=q.device, dtype=dout.dtype))
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)

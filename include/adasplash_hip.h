@@ -121,7 +121,7 @@ size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int d
  *   delta, zinv : [B, Hq, N] fp32 scratch owned by the caller; receive sum_j u_ij dP_ij / sum_j u_ij and
  *                 1 / sum_j p_ij per query row.
  *   alpha, is_causal : 1.5 / 1 for the AdaSplash-2 path, any alpha in (1, 2] for the block-mask path.
- * Rows of dout past a sequence's valid length must be finite (they are multiplied by zero); gradient rows
+ * Rows of q, k, v and dout past a sequence's valid length are never used, whatever they hold; gradient rows
  * past the valid length are written as zeros.  Replaces the four launches at
  * adasplash/adasplash_v2.py:1456-1562 (delta from out2, dq, mask transpose, dk/dv with the GQA group loop)
  * and adasplash/adasplash_block_mask.py:1079-1210.
