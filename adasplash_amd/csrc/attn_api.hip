@@ -20,35 +20,51 @@ int launch_attn_bwd_f32(const AttnBwdParams& p, int D, int am, hipStream_t s);
 //   whatever the caller left in the padding rows never meets an MFMA).
 // With this order a lane of the PV product reads its 8 keys {16s + 4h + r, 16s + 8 + 4h + r} of one
 // d row as one 16-byte LDS access.
+// A thread moves an 8-key x 8-d block: eight 16-byte loads (one key each), an 8 x 8 transpose of 16-bit values in
+// registers (32 byte permutes), eight 16-byte stores (one d row each).  A 64-key tile takes D threads.
 __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
                                                         int N, int Npad, int D, const void* varlen, int varlen_bits,
                                                         int heads) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  uint16_t* tile = reinterpret_cast<uint16_t*>(smem);  // [64][D + 2]
-  const int pitch = D + 2;
-  const int kt = blockIdx.x;
+  const int tiles_per_block = 256 / D;  // D <= 256
+  const int t = threadIdx.x % D;
+  const int kt = blockIdx.x * tiles_per_block + threadIdx.x / D;
+  if (kt >= Npad / 64) return;
   const size_t bh = blockIdx.y;
-  const uint16_t* vsrc = v + bh * (size_t)N * D;
   int L = N;
   if (varlen) {
     const size_t b = bh / heads;
     long long l = varlen_bits == 64 ? ((const long long*)varlen)[b] : (long long)((const int*)varlen)[b];
     L = (int)(l < 0 ? 0 : (l > N ? N : l));
   }
-  for (int i = threadIdx.x; i < 64 * D; i += 256) {
-    int key = i / D, d = i % D;
-    int gk = kt * 64 + key;
-    tile[key * pitch + d] = gk < L ? vsrc[(size_t)gk * D + d] : (uint16_t)0;
+  const int c = t & 7;    // output chunk: positions 8c .. 8c + 7 = keys 16s + 8a + 4h + r, s = c / 2, h = c % 2
+  const int dg = t >> 3;  // d values 8 dg .. 8 dg + 7
+  const uint16_t* vsrc = v + bh * (size_t)N * D + dg * 8;
+  const int key0 = kt * 64 + (c >> 1) * 16 + (c & 1) * 4;
+  u32x4 in[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int gk = key0 + (j >> 2) * 8 + (j & 3);
+    in[j] = u32x4{0u, 0u, 0u, 0u};
+    if (gk < L) in[j] = *reinterpret_cast<const u32x4*>(vsrc + (size_t)gk * D);
   }
-  __syncthreads();
-  uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64 * D;
-  for (int i = threadIdx.x; i < 64 * D; i += 256) {
-    int d = i / 64, pos = i % 64;
-    int key = (pos & ~15) | (((pos >> 2) & 1) << 3) | (((pos >> 3) & 1) << 2) | (pos & 3);
-    vdst[i] = tile[key * pitch + d];
+  uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64 * D + (size_t)(dg * 8) * 64 + c * 8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    u32x4 o;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const uint32_t lo = in[2 * m][e >> 1], hi = in[2 * m + 1][e >> 1];
+      // (e even) low halves, (e odd) high halves of the two keys' dwords, packed key 2m low / key 2m + 1 high
+      o[m] = __builtin_amdgcn_perm(hi, lo, (e & 1) ? 0x07060302u : 0x05040100u);
+    }
+    *reinterpret_cast<u32x4*>(vdst + (size_t)e * 64) = o;
   }
 }
 
+static unsigned vt_layout_blocks(int Npad, int D) {  // 256 / D tiles of 64 keys per block
+  const int tiles = Npad / kBN, per_block = 256 / D;
+  return (unsigned)((tiles + per_block - 1) / per_block);
+}
 static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
 static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }
 static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
@@ -97,8 +113,8 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
     const size_t need = adsp_attn_workspace_bytes(B, Hkv, N, D, dtype);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
     p.vt = workspace;
-    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hkv)), dim3(256),
-                       (size_t)64 * (D + 2) * 2, s, (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3(vt_layout_blocks(p.Npad, D), (unsigned)(B * Hkv)), dim3(256), 0, s,
+                       (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv);
   }
   int rc = dtype == ADSP_BF16 ? launch_attn_bf16(p, D, am, s)
                               : (dtype == ADSP_F16 ? launch_attn_f16(p, D, am, s) : launch_attn_f32(p, D, am, s));
@@ -189,13 +205,13 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     uint16_t* kt = (uint16_t*)workspace;
     uint16_t* qt = kt + (size_t)B * Hkv * D * p.Npad;
     uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
-    const size_t shm = (size_t)64 * (D + 2) * 2;
-    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hkv)), dim3(256), shm, s,
-                       (const uint16_t*)k, kt, N, p.Npad, D, varlen, varlen_bits, Hkv);
-    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hq)), dim3(256), shm, s,
-                       (const uint16_t*)q, qt, N, p.Npad, D, varlen, varlen_bits, Hq);
-    hipLaunchKernelGGL(vt_layout_kernel, dim3((unsigned)(p.Npad / kBN), (unsigned)(B * Hq)), dim3(256), shm, s,
-                       (const uint16_t*)dout, dot, N, p.Npad, D, varlen, varlen_bits, Hq);
+    const unsigned gx = vt_layout_blocks(p.Npad, D);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hkv)), dim3(256), 0, s, (const uint16_t*)k, kt, N, p.Npad, D,
+                       varlen, varlen_bits, Hkv);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, qt, N, p.Npad, D,
+                       varlen, varlen_bits, Hq);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, dot, N, p.Npad,
+                       D, varlen, varlen_bits, Hq);
     p.kt = kt;
     p.qt = qt;
     p.dot = dot;
