@@ -1,7 +1,7 @@
 // Fused sparse entmax attention forward for gfx950 (one kernel: threshold solver + output).
 //
 // Work decomposition
-//   workgroup = 4 waves, owns 128 consecutive query rows of one (batch, head) and is sized so that two
+//   workgroup = 4 waves, owns 128 consecutive query rows of one (batch, head) and is sized so that two to four
 //   workgroups fit a CU; wave w owns rows [32w, 32w+32); inside a wave, lane l holds query row (l & 31)
 //   and, of every 32-key block, the 16 keys {8g + 4(l >> 5) + r : g, r in 0..3} -- the C layout of the
 //   32x32 MFMA when the product is taken as S^T = K Q^T.  All per-row quantities (max, histogram,
@@ -81,7 +81,12 @@ __device__ __forceinline__ void dma16(const void* gsrc, void* lds) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane(base))
-               : "memory", "m0");
+               : "memory");  // (m0 is a reserved register: the compiler sets it itself before each of its own uses)
+}
+
+// 16-byte LDS read at a byte address held as an integer (plus a constant that lands in the instruction's offset field)
+__device__ __forceinline__ u32x4 lds_read16(uint32_t addr, int imm = 0) {
+  return *(const __attribute__((address_space(3))) u32x4*)(addr + imm);
 }
 
 // Tile geometry.  A tile row has kC 16-byte chunks; chunk c of row r is stored at chunk position
@@ -104,15 +109,19 @@ template <typename T, int D> struct TileGeo {
   static constexpr int kVRows = k16 ? D : kBN;
   static constexpr int kVTile = kVRows * kVRow;
   static constexpr int kNBuf = (2 * (kKTile + kVTile) <= 144 * 1024) ? 2 : 1;
-  // Four waves of at most 256 registers: two workgroups share a CU (LDS permitting), one wave of each per
-  // SIMD.  Their barriers are independent, so one workgroup's wait for a tile overlaps the other's MFMAs.
+  // Workgroups of four waves; two to four of them share a CU (registers and LDS permitting), one wave of each
+  // per SIMD.  Their barriers are independent, so one workgroup's wait for a tile overlaps the others' MFMAs.
   static constexpr int kNW = 4;
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
   // Waves per SIMD the register allocation is held to.  The walks are bound by dependent latency, so more
-  // resident waves pay even at the price of a few spills: four for 16-bit D <= 64 (C5 23.3 -> 16.3 ms),
-  // two where the live state needs up to 256 registers, one for the shapes that need more.
-  static constexpr int kMinWaves = (k16 && D <= 64) ? 4 : (((k16 && D <= 128) || (!k16 && D <= 64)) ? 2 : 1);
+  // resident waves pay even at the price of a few spills: four for 16-bit D <= 64 (C5 23.3 -> 16.3 ms), three
+  // for 16-bit D = 128 (168 registers; 12 % fewer cycles than two, part of which the clock gives back), two for
+  // fp32 D <= 64, one for the shapes that need more than 256 registers.
+  // 16-bit D = 128: one V tile instead of two (48 KB of tiles) lets three workgroups share a CU; the output walk
+  // then loads a tile's V while its scores are computed and waits for it before the first PV product.
+  static constexpr bool kVSingle = k16 && D == 128;
+  static constexpr int kMinWaves = (k16 && D <= 64) ? 4 : (kVSingle ? 3 : ((!k16 && D <= 64) ? 2 : 1));
   static constexpr int kQRegs = k16 ? (D / 16) * 4 : D / 2;  // dwords of Q held per lane
   static constexpr int kDB = D >= 32 ? D / 32 : 1;           // 32-wide d blocks of the output
   static constexpr int kKLoads = kKTile / 1024;              // wave-level 1 KB DMA instructions per K tile
@@ -143,10 +152,13 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   __shared__ __align__(1024) unsigned char k_lds0[G::kKTile];
   __shared__ __align__(1024) unsigned char v_lds0[G::kVTile];
   __shared__ __align__(1024) unsigned char k_lds1[G::kNBuf == 2 ? G::kKTile : 16];
-  __shared__ __align__(1024) unsigned char v_lds1[G::kNBuf == 2 ? G::kVTile : 16];
-  __shared__ uint32_t mask_a[kMaskWords];
-  __shared__ uint32_t mask_b[kMaskWords];
-  __shared__ uint32_t mask_out[2][kMaskWords];  // per 128-row half of the row block, for the bmask output
+  __shared__ __align__(1024) unsigned char v_lds1[(G::kNBuf == 2 && !G::kVSingle) ? G::kVTile : 16];
+  // tile masks, sized by the launch for this problem's number of key tiles (4 x mask_words words of dynamic LDS):
+  // two that the walks read and write in turn, and one per 128-row half of the row block for the bmask output
+  extern __shared__ uint32_t mask_pool[];
+  uint32_t* const mask_a = mask_pool;
+  uint32_t* const mask_b = mask_pool + p.mask_words;
+  uint32_t* const mask_out0 = mask_pool + 2 * p.mask_words;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
@@ -258,6 +270,13 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     const int row = P / VS::kC;
     voff[j0] = (uint32_t)(row * G::kVRow + (((P % VS::kC) ^ VS::sw(row)) << 4));
   }
+  // Swizzled read addresses without a register per fragment (three waves per SIMD leave none to spare): chunk c
+  // of row r sits at r * row_bytes + ((c ^ sw(r)) << 4), and with c = 2 ks + lh that is
+  // (r * row_bytes + ((lh ^ sw(r)) << 4)) ^ (ks << 5) -- one lane constant and one xor with an immediate per
+  // read.  Rows r and r + 32 share sw, so the second key block is an offset.  Same for the V^T tile with
+  // c = 4 kb + 2 s + lh.
+  const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
+  const uint32_t v_lane = (uint32_t)(lq * G::kVRow + ((lh ^ VS::sw(lq)) << 4));
   auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKPer], unsigned char* lds, int kt) {
     // a row-major [64][D] tile out of a row-major tensor (K, or V for fp32); the last tile may stick out
     const unsigned char* base = g + (size_t)kt * G::kKTile;
@@ -319,9 +338,41 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
 
   // Runs body(kt, k_tile, v_tile) over the selected tiles; the DMA of the next tile is issued right
   // after the barrier that publishes the current one and completes under the current tile's MFMAs.
+  bool k_after_v = false;  // single V tile: a K tile's loads were issued after the current V tile's
   auto tile_loop = [&](const uint32_t* mask, bool with_v, auto&& body) {
     __syncthreads();  // the previous pass is done with the LDS tiles; its mask writes are visible
     mw_index = -1;
+    if constexpr (G::kVSingle) {
+      if (with_v) {
+        // K double-buffered, V single: the barrier that publishes K(t) also says every wave is done with V(t-1);
+        // V(t) is then loaded under the score product of tile t and the body waits for it (a second barrier)
+        // before its first PV product.
+        int cur = next_tile(mask, -1);
+        if (cur >= 0) issue_k(k_lds0, cur);
+        while (cur >= 0) {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+          __syncthreads();
+          int nxt = next_tile(mask, cur);
+          issue_v(v_lds0, cur);
+          if (nxt >= 0) issue_k(k_lds1, nxt);
+          k_after_v = nxt >= 0;
+          __builtin_amdgcn_sched_barrier(0);
+          body(cur, k_lds0, v_lds0);
+          cur = nxt;
+          if (cur < 0) break;
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+          __syncthreads();
+          nxt = next_tile(mask, cur);
+          issue_v(v_lds0, cur);
+          if (nxt >= 0) issue_k(k_lds0, nxt);
+          k_after_v = nxt >= 0;
+          __builtin_amdgcn_sched_barrier(0);
+          body(cur, k_lds1, v_lds0);
+          cur = nxt;
+        }
+        return;
+      }
+    }
     int cur = next_tile(mask, -1);
     if (cur >= 0) {
       issue_k(k_lds0, cur);
@@ -375,7 +426,25 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     const unsigned char* krow0 = kt_lds + lq * G::kKRow;
     const unsigned char* krow1 = kt_lds + (32 + lq) * G::kKRow;
     const int sw0 = KS::sw(lq), sw1 = KS::sw(32 + lq);
-    if constexpr (k16) {
+    if constexpr (k16 && G::kVSingle) {
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
+      asm volatile("" : "+v"(ka));  // keeps the eight xors here instead of eight registers hoisted out of the walk
+      u32x4 a0[D / 16], a1[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a0[ks] = lds_read16(ka ^ (ks << 5));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a1[ks] = lds_read16(ka ^ (ks << 5), 32 * G::kKRow);
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s0 = mfma_16bit<T>(a0[ks], bq, s0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s1 = mfma_16bit<T>(a1[ks], bq, s1);
+      }
+    } else if constexpr (k16) {
       u32x4 a0[D / 16], a1[D / 16];
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) a0[ks] = *reinterpret_cast<const u32x4*>(krow0 + (((2 * ks + lh) ^ sw0) << 4));
@@ -413,7 +482,23 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     const int row = kb * 32 + lq;
     const unsigned char* krow = kt_lds + row * G::kKRow;
     const int sw = KS::sw(row);
-    if constexpr (k16) {
+    if constexpr (k16 && G::kVSingle) {
+      // register budget of three waves per SIMD: the K fragments are fetched four at a time
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
+      asm volatile("" : "+v"(ka));
+#pragma unroll
+      for (int k0 = 0; k0 < D / 16; k0 += 4) {
+        u32x4 a[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) a[ks] = lds_read16(ka ^ ((k0 + ks) << 5), kb * 32 * G::kKRow);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          u32x4 bq = {qf[(k0 + ks) * 4], qf[(k0 + ks) * 4 + 1], qf[(k0 + ks) * 4 + 2], qf[(k0 + ks) * 4 + 3]};
+          acc = mfma_16bit<T>(a[ks], bq, acc);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else if constexpr (k16) {
       u32x4 a[D / 16];
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(krow + (((2 * ks + lh) ^ sw) << 4));
@@ -474,12 +559,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   };
   auto mark_tile = [&](uint32_t* mask, int kt) { atomicOr(&mask[kt >> 5], 1u << (kt & 31)); };
 
-  for (int i = tid; i < kMaskWords; i += G::kThreads) {
-    mask_a[i] = 0u;
-    mask_b[i] = 0u;
-    mask_out[0][i] = 0u;
-    mask_out[1][i] = 0u;
-  }
+  for (int i = tid; i < 4 * p.mask_words; i += G::kThreads) mask_pool[i] = 0u;
 
   // ---- pass A (+B): row max, and for alpha = 1.5 / 2 the histogram bracket in the same walk ----------------
   uint32_t* mask_cur = nullptr;  // mask consumed by the next pass
@@ -743,7 +823,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
         __syncthreads();
         mask_cur = mask_new;
         mask_new = (mask_cur == mask_a) ? mask_b : mask_a;
-        for (int i = tid; i < kMaskWords; i += G::kThreads) mask_new[i] = 0u;
+        for (int i = tid; i < p.mask_words; i += G::kThreads) mask_new[i] = 0u;
       }
     }
   }
@@ -765,6 +845,19 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     const float init = -tau * inv_qs;
     tile_loop(mask_cur, true, [&](int kt, const unsigned char* kt_lds, const unsigned char* vt_lds) {
       bool tile_active = false;
+      // single V tile: every wave joins one barrier per tile once its own share of V has landed (the K loads of
+      // the next tile, issued after it, may still be in flight), whether or not it has work in the tile
+      bool v_ready = !G::kVSingle;
+      auto need_v = [&]() {
+        if constexpr (G::kVSingle) {
+          if (!v_ready) {
+            if (k_after_v) __builtin_amdgcn_s_waitcnt(0x0f70 | kKPer);  // vmcnt(kKPer)
+            else __builtin_amdgcn_s_waitcnt(0x0f70);
+            __syncthreads();
+            v_ready = true;
+          }
+        }
+      };
       for_tile_blocks(kt, kt_lds, init, [&](const f32x16& acc, int kb) {
         float pv[16];
         float bsum = 0.f;
@@ -790,7 +883,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           const unsigned long long q0 = 0x0000ffff0000ffffull, q1 = 0xffff0000ffff0000ull;
           active16 += ((blo & q0) != 0) + ((blo & q1) != 0) + ((bhi & q0) != 0) + ((bhi & q1) != 0);
         }
+        need_v();
         if constexpr (k16) {
+          uint32_t va = (uint32_t)(uintptr_t)vt_lds + v_lane;
+          asm volatile("" : "+v"(va));
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
             u32x4 bp = {pack2<T>(pv[8 * s], pv[8 * s + 1]), pack2<T>(pv[8 * s + 2], pv[8 * s + 3]),
@@ -799,8 +895,12 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
             for (int db = 0; db < G::kDB; ++db) {
               const int drow = db * 32 + lq;
               u32x4 a = {0u, 0u, 0u, 0u};
-              if (D >= 32 || drow < D)
-                a = *reinterpret_cast<const u32x4*>(vt_lds + VS::off(drow, kb * 4 + 2 * s + lh));
+              if constexpr (G::kVSingle) {
+                a = lds_read16(va ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
+              } else {
+                if (D >= 32 || drow < D)
+                  a = *reinterpret_cast<const u32x4*>(vt_lds + VS::off(drow, kb * 4 + 2 * s + lh));
+              }
               o[db] = mfma_16bit<T>(a, bp, o[db]);
             }
           }
@@ -820,9 +920,10 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           }
         }
       });
+      need_v();
       // final block mask: tiles in which this 128-row half really has a non-zero probability
       if (bmask_out && __builtin_amdgcn_ballot_w64(tile_active && qi < L) != 0ull && lane == 0)
-        mark_tile(mask_out[half], kt);
+        mark_tile(mask_out0 + half * p.mask_words, kt);
     });
   }
   psum += __shfl_xor(psum, 32, 64);
@@ -883,7 +984,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     __syncthreads();
     for (int i = tid; i < kHalves * p.mask_words; i += G::kThreads) {
       const int hf = i / p.mask_words, w = i % p.mask_words;
-      if (m0 + hf * kMaskRows < N) bmask_out[i] = (int32_t)mask_out[hf][w];
+      if (m0 + hf * kMaskRows < N) bmask_out[i] = (int32_t)mask_out0[hf * p.mask_words + w];
     }
   }
 }

@@ -11,7 +11,7 @@ template <typename T, int D, int AM> static int launch_attn_one(const AttnParams
   const long long n_mblk = (p.N + G::kBM - 1) / G::kBM;
   const long long total = (long long)p.B * p.Hkv * n_mblk * group;
   const long long per_xcd = (total + 7) / 8;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(G::kThreads), 0, s, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(G::kThreads), (size_t)4 * p.mask_words * sizeof(uint32_t), s, p);  // dynamic LDS: the tile masks
   return 0;
 }
 
