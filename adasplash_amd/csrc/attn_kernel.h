@@ -270,7 +270,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     const int row = P / VS::kC;
     voff[j0] = (uint32_t)(row * G::kVRow + (((P % VS::kC) ^ VS::sw(row)) << 4));
   }
-  // Swizzled read addresses without a register per fragment (three waves per SIMD leave none to spare): chunk c
+  // Swizzled read addresses without a register per fragment (three or four waves per SIMD leave none to spare): chunk c
   // of row r sits at r * row_bytes + ((c ^ sw(r)) << 4), and with c = 2 ks + lh that is
   // (r * row_bytes + ((lh ^ sw(r)) << 4)) ^ (ks << 5) -- one lane constant and one xor with an immediate per
   // read.  Rows r and r + 32 share sw, so the second key block is an offset.  Same for the V^T tile with
@@ -426,7 +426,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     const unsigned char* krow0 = kt_lds + lq * G::kKRow;
     const unsigned char* krow1 = kt_lds + (32 + lq) * G::kKRow;
     const int sw0 = KS::sw(lq), sw1 = KS::sw(32 + lq);
-    if constexpr (k16 && G::kVSingle) {
+    if constexpr (k16) {
       uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
       asm volatile("" : "+v"(ka));  // keeps the eight xors here instead of eight registers hoisted out of the walk
       u32x4 a0[D / 16], a1[D / 16];
@@ -434,22 +434,6 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       for (int ks = 0; ks < D / 16; ++ks) a0[ks] = lds_read16(ka ^ (ks << 5));
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) a1[ks] = lds_read16(ka ^ (ks << 5), 32 * G::kKRow);
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
-        s0 = mfma_16bit<T>(a0[ks], bq, s0);
-      }
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
-        s1 = mfma_16bit<T>(a1[ks], bq, s1);
-      }
-    } else if constexpr (k16) {
-      u32x4 a0[D / 16], a1[D / 16];
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) a0[ks] = *reinterpret_cast<const u32x4*>(krow0 + (((2 * ks + lh) ^ sw0) << 4));
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) a1[ks] = *reinterpret_cast<const u32x4*>(krow1 + (((2 * ks + lh) ^ sw1) << 4));
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
         u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
@@ -499,9 +483,11 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
         __builtin_amdgcn_sched_barrier(0);
       }
     } else if constexpr (k16) {
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
+      asm volatile("" : "+v"(ka));
       u32x4 a[D / 16];
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(krow + (((2 * ks + lh) ^ sw) << 4));
+      for (int ks = 0; ks < D / 16; ++ks) a[ks] = lds_read16(ka ^ (ks << 5), kb * 32 * G::kKRow);
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
         u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
@@ -895,12 +881,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
             for (int db = 0; db < G::kDB; ++db) {
               const int drow = db * 32 + lq;
               u32x4 a = {0u, 0u, 0u, 0u};
-              if constexpr (G::kVSingle) {
-                a = lds_read16(va ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
-              } else {
-                if (D >= 32 || drow < D)
-                  a = *reinterpret_cast<const u32x4*>(vt_lds + VS::off(drow, kb * 4 + 2 * s + lh));
-              }
+              if (D >= 32 || drow < D) a = lds_read16(va ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
               o[db] = mfma_16bit<T>(a, bp, o[db]);
             }
           }
