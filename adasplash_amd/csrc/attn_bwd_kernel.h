@@ -105,6 +105,8 @@ template <typename T, int D> struct BwdTiles {
     }
   }
   // acc[i] = (tile row kb*32 + 8(i/4) + 4 lh + i%4) . (lane's row), for the 32 lane rows of the wave.
+  // kLean: addresses by xor with immediates (fewer registers, a few more VALU instructions) -- see below.
+  template <bool kLean = false>
   static __device__ __forceinline__ f32x16 dot_block(const unsigned char* tile, int kb, const uint32_t (&f)[G::kQRegs],
                                                      int lq, int lh) {
     f32x16 acc;
@@ -113,10 +115,25 @@ template <typename T, int D> struct BwdTiles {
     const int row = kb * 32 + lq;
     const unsigned char* trow = tile + row * G::kKRow;
     const int sw = KS::sw(row);
-    if constexpr (k16) {
+    if constexpr (k16 && !kLean) {
       u32x4 a[D / 16];
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(trow + (((2 * ks + lh) ^ sw) << 4));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 b = {f[ks * 4], f[ks * 4 + 1], f[ks * 4 + 2], f[ks * 4 + 3]};
+        acc = mfma_16bit<T>(a[ks], b, acc);
+      }
+    } else if constexpr (k16) {
+      // chunk 2 ks + lh of row r sits at r * row_bytes + (((2 ks + lh) ^ sw(r)) << 4)
+      //   = (r * row_bytes + ((lh ^ sw(r)) << 4)) ^ (ks << 5): one lane constant, an xor with an immediate per read
+      // (rows r and r + 32 share sw, so the block is an offset); the empty asm keeps the xors here instead of a
+      // register per fragment hoisted out of the walk
+      uint32_t ta = (uint32_t)(uintptr_t)tile + (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
+      asm volatile("" : "+v"(ta));
+      u32x4 a[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a[ks] = lds_read16(ta ^ (ks << 5), kb * 32 * G::kKRow);
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
         u32x4 b = {f[ks * 4], f[ks * 4 + 1], f[ks * 4 + 2], f[ks * 4 + 3]};
@@ -137,9 +154,10 @@ template <typename T, int D> struct BwdTiles {
   // w holds the lane's 16 values in the accumulator order of dot_block.  16-bit: `tile` is the transposed
   // tile (its padding rows are zero); fp32: the row-major one, of which only the first `rows_valid` rows
   // are used (padding rows of the caller's tensors may hold anything).
+  template <bool kLean = false>
   static __device__ __forceinline__ void acc_block(f32x16 (&o)[G::kDB], const unsigned char* tile, int kb,
                                                    const float (&w)[16], int lq, int lh, int rows_valid) {
-    if constexpr (k16) {
+    if constexpr (k16 && !kLean) {
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         u32x4 b = {pack2<T>(w[8 * s], w[8 * s + 1]), pack2<T>(w[8 * s + 2], w[8 * s + 3]),
@@ -149,6 +167,22 @@ template <typename T, int D> struct BwdTiles {
           const int drow = db * 32 + lq;
           u32x4 a = {0u, 0u, 0u, 0u};
           if (D >= 32 || drow < D) a = *reinterpret_cast<const u32x4*>(tile + VS::off(drow, kb * 4 + 2 * s + lh));
+          o[db] = mfma_16bit<T>(a, b, o[db]);
+        }
+      }
+    } else if constexpr (k16) {
+      // same addressing for the transposed tile: chunk 4 kb + 2 s + lh of row 32 db + lq
+      uint32_t ta = (uint32_t)(uintptr_t)tile + (uint32_t)(lq * G::kVRow + ((lh ^ VS::sw(lq)) << 4));
+      asm volatile("" : "+v"(ta));
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        u32x4 b = {pack2<T>(w[8 * s], w[8 * s + 1]), pack2<T>(w[8 * s + 2], w[8 * s + 3]),
+                   pack2<T>(w[8 * s + 4], w[8 * s + 5]), pack2<T>(w[8 * s + 6], w[8 * s + 7])};
+#pragma unroll
+        for (int db = 0; db < G::kDB; ++db) {
+          const int drow = db * 32 + lq;
+          u32x4 a = {0u, 0u, 0u, 0u};
+          if (D >= 32 || drow < D) a = lds_read16(ta ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
           o[db] = mfma_16bit<T>(a, b, o[db]);
         }
       }
@@ -233,8 +267,16 @@ __device__ __forceinline__ bool bwd_block_map(int units, int inner, int& unit, i
 // ---------------------------------------------------------------------------------------------------------
 // dQ kernel: one block per (K/V head, query head in its group, row block of 128 queries)
 // ---------------------------------------------------------------------------------------------------------
+#ifndef ADSP_DQ_PLAIN_MAXD
+#define ADSP_DQ_PLAIN_MAXD 128
+#endif
+#ifndef ADSP_DQ_WAVES64
+#define ADSP_DQ_WAVES64 3
+#endif
+template <typename T, int D> constexpr int dq_waves() { return (TileGeo<T, D>::k16 && D <= 64) ? ADSP_DQ_WAVES64 : BwdTiles<T, D>::kMinWaves; }
+
 template <typename T, int D, int AM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T, D>::kMinWaves), 2))) void attn_bwd_dq_kernel(AttnBwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T, D>()), (dq_waves<T, D>() > 2 ? dq_waves<T, D>() : 2)))) void attn_bwd_dq_kernel(AttnBwdParams p) {
   using BT = BwdTiles<T, D>;
   using G = TileGeo<T, D>;
   constexpr bool k16 = G::k16;
@@ -347,12 +389,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   // one fma per score instead of a compare and two selects more.  The choice is a template argument so that each
   // kind of block is one piece of straight-line code, products included.
   // (only where the second code path fits the register budget: at D = 128 it costs spills and more than it saves)
-  constexpr bool kPlainBlocks = k16 && D <= 64;
+  constexpr bool kPlainBlocks = k16 && D <= ADSP_DQ_PLAIN_MAXD;
   auto block_is_plain = [&](int kt, int kb) { return kPlainBlocks && kt * kBN + kb * 32 + 31 <= lim_all; };
   auto block_terms = [&](auto plain_c, int kt, int kb, const unsigned char* ka, const unsigned char* va, float (&r)[16],
                          f32x16& dp) {
-    f32x16 s = BT::dot_block(ka, kb, qf, lq, lh);
-    dp = BT::dot_block(va, kb, dof, lq, lh);
+    f32x16 s = BT::template dot_block<true>(ka, kb, qf, lq, lh);
+    dp = BT::template dot_block<true>(va, kb, dof, lq, lh);
     if constexpr (decltype(plain_c)::value) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) r[i] = fmaf(s[i], p.qscale, -tau);
@@ -429,7 +471,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
           bwd_prob<AM>(r[i], p.c0, pr, u);
           dx[i] = u * (dp[i] - delta);
         }
-        BT::acc_block(acc, k16 ? kta : ka, kb, dx, lq, lh, L - kt * kBN);
+        BT::template acc_block<true>(acc, k16 ? kta : ka, kb, dx, lq, lh, L - kt * kBN);
       };
       if constexpr (!kPlainBlocks) {
         block(std::false_type{});
