@@ -846,12 +846,13 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       };
       for_tile_blocks(kt, kt_lds, init, [&](const f32x16& acc, int kb) {
         float pv[16];
-        float bsum = 0.f;
+        float hsum[2] = {0.f, 0.f};  // over the lane's keys of each 16-key half of the block
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           pv[i] = attn_prob<AM>(acc[i], qs, p.c0);
-          bsum += pv[i];
+          hsum[i >> 3] += pv[i];
         }
+        const float bsum = hsum[0] + hsum[1];
         psum += bsum;
         tile_active |= bsum > 0.f;
         if (p.tile_counts) {
@@ -875,6 +876,9 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           asm volatile("" : "+v"(va));
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
+            // a 16-key half in which no row of the wave has a non-zero probability adds nothing: with a
+            // support of a few keys per row that is a large share of the halves
+            if (__builtin_amdgcn_ballot_w64(hsum[s] > 0.f) == 0ull) continue;
             u32x4 bp = {pack2<T>(pv[8 * s], pv[8 * s + 1]), pack2<T>(pv[8 * s + 2], pv[8 * s + 3]),
                         pack2<T>(pv[8 * s + 4], pv[8 * s + 5]), pack2<T>(pv[8 * s + 6], pv[8 * s + 7])};
 #pragma unroll
