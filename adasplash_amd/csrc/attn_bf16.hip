@@ -1,5 +1,8 @@
-// attn_fwd_kernel instantiations for element type bf16_t.
+// attn_fwd_kernel instantiations for element type bf16_t: no or one solver step.
 #include "attn_launch.h"
 namespace adsp {
-int launch_attn_bf16(const AttnParams& p, int D, int am, hipStream_t s) { return launch_attn<bf16_t>(p, D, am, s); }
+int launch_attn_multi_bf16(const AttnParams& p, int D, int am, hipStream_t s);
+int launch_attn_bf16(const AttnParams& p, int D, int am, hipStream_t s) {
+  return p.niter >= 2 ? launch_attn_multi_bf16(p, D, am, s) : launch_attn<bf16_t, false>(p, D, am, s);
+}
 }  // namespace adsp

@@ -1,5 +1,8 @@
-// attn_fwd_kernel instantiations for element type float.
+// attn_fwd_kernel instantiations for element type float: no or one solver step.
 #include "attn_launch.h"
 namespace adsp {
-int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s) { return launch_attn<float>(p, D, am, s); }
+int launch_attn_multi_f32(const AttnParams& p, int D, int am, hipStream_t s);
+int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s) {
+  return p.niter >= 2 ? launch_attn_multi_f32(p, D, am, s) : launch_attn<float, false>(p, D, am, s);
+}
 }  // namespace adsp

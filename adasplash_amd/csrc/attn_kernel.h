@@ -26,6 +26,7 @@
 // The 16-bit path consumes V through a tile-wise key-major copy (vt_layout_kernel) so that the PV product
 // out^T = V^T P^T can take P^T straight from the S^T accumulators without an LDS round trip.
 #pragma once
+#include <type_traits>
 #include "common.h"
 #include "solver.h"
 #include "attn_params.h"
@@ -114,6 +115,8 @@ template <typename T, int D> struct TileGeo {
   static constexpr int kNW = 4;
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
+  // words of dynamic LDS after the tile masks: the waves' chunk counters and two flags
+  static constexpr int kPoolTail = kNW + 2;
   // Waves per SIMD the register allocation is held to.  The walks are bound by dependent latency, so more
   // resident waves pay even at the price of a few spills: four for 16-bit D <= 64 (C5 23.3 -> 16.3 ms), three
   // for 16-bit D = 128 (168 registers; 12 % fewer cycles than two, part of which the clock gives back), two for
@@ -139,7 +142,9 @@ template <int AM> __device__ __forceinline__ float attn_prob(float r, float qs, 
   return r > 0.f ? fast_exp2(fast_log2(r * qs) * c0) : 0.f;
 }
 
-template <typename T, int D, int AM>
+// kMulti: the instance for two and more solver steps, which carries the candidate lists of the solver walks; the
+// other one (no or one step) does not pay for their registers.
+template <typename T, int D, int AM, bool kMulti>
 __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_waves_per_eu(TileGeo<T, D>::kMinWaves, (TileGeo<T, D>::kMinWaves > 2 ? TileGeo<T, D>::kMinWaves : 2)))) void attn_fwd_kernel(AttnParams p) {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
@@ -154,11 +159,22 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   __shared__ __align__(1024) unsigned char k_lds1[G::kNBuf == 2 ? G::kKTile : 16];
   __shared__ __align__(1024) unsigned char v_lds1[(G::kNBuf == 2 && !G::kVSingle) ? G::kVTile : 16];
   // tile masks, sized by the launch for this problem's number of key tiles (4 x mask_words words of dynamic LDS):
-  // two that the walks read and write in turn, and one per 128-row half of the row block for the bmask output
+  // two that the walks read and write in turn, and one per 128-row half of the row block for the bmask output.
+  // With p.fine_masks another 2 x kNW x 2 x mask_words words follow: for each of the two walk masks and each
+  // wave, one bit per 32-key block (bit 2 kt + kb) saying whether that wave's 32 rows need the block.
   extern __shared__ uint32_t mask_pool[];
   uint32_t* const mask_a = mask_pool;
   uint32_t* const mask_b = mask_pool + p.mask_words;
   uint32_t* const mask_out0 = mask_pool + 2 * p.mask_words;
+  constexpr bool kFine = kMulti;  // the walks of a single step gain too little from them
+  uint32_t* const fine_pool = kFine && p.fine_masks ? mask_pool + 4 * p.mask_words : nullptr;
+  // after the masks, the bookkeeping of the candidate lists (see the solver walks): a chunk counter per wave and
+  // two flag words
+  constexpr int kPoolTail = G::kPoolTail;
+  static_assert(kPoolTail == NW + 2, "launch and kernel disagree on the LDS tail");
+  const int mask_pool_words = (p.fine_masks ? 4 + 4 * G::kNW : 4) * p.mask_words;
+  uint32_t* const chunk_ctr = mask_pool + mask_pool_words;
+  uint32_t* const list_flag = chunk_ctr + NW;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
@@ -318,6 +334,21 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   // a register, so LDS is read once per 32 tiles.
   int mw_index = -1;
   uint32_t mw_bits = 0u;
+  // this wave's block bits of a walk mask (null: every block), and the pair of bits of tile kt, cached 16 tiles a word
+  auto fine_of = [&](const uint32_t* mask) -> uint32_t* {
+    if (!fine_pool || !mask) return nullptr;
+    return fine_pool + ((mask == mask_a ? 0 : G::kNW) + wave) * 2 * p.mask_words;
+  };
+  int fw_index = -1;
+  uint32_t fw_bits = 0u;
+  auto block_bits = [&](const uint32_t* fine, int kt) -> uint32_t {
+    if (!fine) return 3u;
+    if ((kt >> 4) != fw_index) {
+      fw_index = kt >> 4;
+      fw_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)fine[fw_index]);
+    }
+    return (fw_bits >> ((kt & 15) * 2)) & 3u;
+  };
   auto next_tile = [&](const uint32_t* mask, int cur) -> int {
     int t = cur + 1;
     if (!mask) return t < nt ? t : -1;
@@ -342,6 +373,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   auto tile_loop = [&](const uint32_t* mask, bool with_v, auto&& body) {
     __syncthreads();  // the previous pass is done with the LDS tiles; its mask writes are visible
     mw_index = -1;
+    fw_index = -1;
     if constexpr (G::kVSingle) {
       if (with_v) {
         // K double-buffered, V single: the barrier that publishes K(t) also says every wave is done with V(t-1);
@@ -532,28 +564,74 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     }
   };
   // Block-by-block variant: f(s, kb) per visible 32-key block.
-  auto for_tile_blocks = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
+  auto for_tile_blocks = [&](int kt, const unsigned char* kt_lds, float init, uint32_t bits, auto&& f) {
     if (p.causal && kt * kBN > wave_row0 + 31) return;
     const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-      if (p.causal && kt * kBN + kb * 32 > wave_row0 + 31) continue;
+      if (!((bits >> kb) & 1u) || (p.causal && kt * kBN + kb * 32 > wave_row0 + 31)) continue;
       f32x16 acc = block_scores(kt_lds, kb, init);
       if (need_mask) mask_block(acc, kt, kb);
       f(acc, kb);
     }
   };
+  // Per-block variant for the walks that follow a mask: f(s, kb) for the blocks of tile kt named by `bits`
+  // (bit kb).  Both blocks take the two-chain code of for_tile; a single block takes one chain.
+  auto for_tile_sel = [&](int kt, const unsigned char* kt_lds, float init, uint32_t bits, auto&& f) {
+    if (bits == 0u || (p.causal && kt * kBN > wave_row0 + 31)) return;
+    const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
+    if (bits == 3u) {
+      f32x16 s0, s1;
+      if (need_mask) {
+        asm volatile("; masked tile" ::: "memory");
+        tile_scores(kt_lds, init, s0, s1);
+        mask_block(s0, kt, 0);
+        mask_block(s1, kt, 1);
+        f(s0, 0);
+        f(s1, 1);
+      } else {
+        asm volatile("; plain tile" ::: "memory");
+        tile_scores(kt_lds, init, s0, s1);
+        f(s0, 0);
+        f(s1, 1);
+      }
+    } else if (bits == 1u) {
+      asm volatile("; block 0" ::: "memory");
+      f32x16 acc = block_scores(kt_lds, 0, init);
+      if (need_mask) mask_block(acc, kt, 0);
+      f(acc, 0);
+    } else {
+      asm volatile("; block 1" ::: "memory");
+      f32x16 acc = block_scores(kt_lds, 1, init);
+      if (need_mask) mask_block(acc, kt, 1);
+      f(acc, 1);
+    }
+  };
   auto mark_tile = [&](uint32_t* mask, int kt) { atomicOr(&mask[kt >> 5], 1u << (kt & 31)); };
+  // one lane of a wave: the tile for the row block, and the wave's own blocks `bits` of it
+  auto mark_blocks = [&](uint32_t* mask, uint32_t* fine, int kt, uint32_t bits) {
+    atomicOr(&mask[kt >> 5], 1u << (kt & 31));
+    if (fine) atomicOr(&fine[kt >> 4], bits << ((kt & 15) * 2));
+  };
+  auto clear_mask = [&](uint32_t* mask) {  // by every thread of the block
+    for (int i = tid; i < p.mask_words; i += G::kThreads) mask[i] = 0u;
+    if (fine_pool) {
+      uint32_t* f = fine_pool + (mask == mask_a ? 0 : G::kNW) * 2 * p.mask_words;
+      for (int i = tid; i < G::kNW * 2 * p.mask_words; i += G::kThreads) f[i] = 0u;
+    }
+  };
 
-  for (int i = tid; i < 4 * p.mask_words; i += G::kThreads) mask_pool[i] = 0u;
+  for (int i = tid; i < mask_pool_words + kPoolTail; i += G::kThreads) mask_pool[i] = 0u;
 
   // ---- pass A (+B): row max, and for alpha = 1.5 / 2 the histogram bracket in the same walk ----------------
   uint32_t* mask_cur = nullptr;  // mask consumed by the next pass
   uint32_t* mask_new = mask_a;   // mask produced by the running pass
+  uint32_t* fine_new = fine_of(mask_new);
   const int half = (wave * 32) / kMaskRows;  // which 128-row half of the row block this wave belongs to
   const bool with_hist = AM != ATT_GEN && p.use_hist;
   float m_raw = -INFINITY;
   float hist_lo = 0.f;  // lower bound of tau from the histogram (valid when with_hist)
+  float cand_est = 0.f;  // with the histogram: how many scores of this wave's rows may lie above that bound
   constexpr float kBinW = 1.f / (float)kAttnBins;  // bin width in z units
   if (!with_hist) {
     tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
@@ -591,7 +669,6 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     // window coordinate y = s c8 - g0 + 1: [0, 1) below the window, [i, i + 1) at bit position i; the
     // conversion rounds, hence the half
     float offn = (0.5f - (float)g0) * (1.f / 65535.f);
-    uint32_t live2 = 0u;  // bit positions of the nine bins under the running maximum, in both halves
     // moves the window up by sh bins (per lane, sh >= 0)
     auto shift_planes = [&](int sh) {
       const uint32_t s1 = (uint32_t)(sh < 15 ? sh : 15);
@@ -600,12 +677,22 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       for (int k = 0; k < kPlanes; ++k) pl[k] = pk_shr16(pl[k], s2);
     };
     tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
-      bool any = false;
+      bool any0 = false, any1 = false;
       for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
-        float tm = m_raw;
+        float tm0 = s0[0], tm1 = s1[0];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) tm = fmaxf(fmaxf(tm, s0[i]), s1[i]);
-        m_raw = tm;
+        for (int i = 1; i < 16; ++i) {
+          tm0 = fmaxf(tm0, s0[i]);
+          tm1 = fmaxf(tm1, s1[i]);
+        }
+        m_raw = fmaxf(m_raw, fmaxf(tm0, tm1));
+        {
+          // a block matters to the later walks when one of its entries lies within 1 (in z) of the running
+          // maximum; the margin covers the rounding of the difference
+          const float keep = m_raw - inv_qs * 1.0001f - 1e-6f * fabsf(m_raw);
+          any0 = tm0 > keep;
+          any1 = tm1 > keep;
+        }
         // bin of the maximum; the entries use the same scale, so none lands more than a rounding error above it
         const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : g0 + kTopLo - 1;
         int p_top = g_top - g0 + 1;
@@ -616,10 +703,6 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           p_top -= sh;
           offn = (0.5f - (float)g0) * (1.f / 65535.f);
         }
-        {
-          const uint32_t lo = (uint32_t)(p_top - kAttnBins);
-          live2 = pk_shl16(0xffffffffu, lo | (lo << 16));
-        }
         uint32_t w[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
@@ -627,10 +710,6 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           const float sb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
           w[j] = pk_shl16(0x00010001u, __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_u16(fmaf(sa, c8n, offn), fmaf(sb, c8n, offn))));
         }
-        uint32_t seen = 0u;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) seen |= w[j];
-        any = (seen & live2) != 0u;  // some entry of the tile lies within 1 of the running maximum
         // adder tree: 16 words + plane 0 -> plane 0 and 8 carries, those + plane 1 -> plane 1 and 4 carries, ...
         uint32_t c2[8], c4[4], c8w[2], c16;
         uint32_t acc = pl[0];
@@ -666,7 +745,12 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           }
         }
       });
-      if (__builtin_amdgcn_ballot_w64(any) != 0ull && lane == 0) mark_tile(mask_new, kt);
+      if constexpr (kFine) {
+        const uint32_t nb = (__builtin_amdgcn_ballot_w64(any0) != 0ull ? 1u : 0u) | (__builtin_amdgcn_ballot_w64(any1) != 0ull ? 2u : 0u);
+        if (nb && lane == 0) mark_blocks(mask_new, fine_new, kt, nb);
+      } else {
+        if (__builtin_amdgcn_ballot_w64(any0 || any1) != 0ull && lane == 0) mark_tile(mask_new, kt);
+      }
     });
     // the two lanes of a row bring their windows to the row's nine bins, bin g_top - 8 at bit position 1; then
     // the counters are read out of the planes (both halves of a word belong to the lane's row) and added up
@@ -692,8 +776,15 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     // less than one bin width off (the entries left out lie below max - 1).
     const float t_shift = (float)g0_row * kBinW;
     hist_lo = (AM == ATT_15) ? hist_bracket_alpha15<W>(cnt, t_shift, kBinW) : hist_bracket_alpha2<W>(cnt, t_shift, kBinW);
+    {
+      float n_cand = 0.f;  // the entries of the bins that reach above the bound
+#pragma unroll
+      for (int k = 0; k < W; ++k) n_cand += (t_shift + (float)(k + 1) * kBinW > hist_lo) ? cnt[k] : 0.f;
+      cand_est = wave_sum(lh == 0 && qi < L ? n_cand : 0.f);
+    }
     mask_cur = mask_new;
     mask_new = mask_b;
+    fine_new = fine_of(mask_new);
   }
   const float m = m_raw * qs;  // row max of z = (alpha-1) q.k / sqrt(D)
 
@@ -718,31 +809,112 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   return;
 #endif
   // ---- pass C: niter safeguarded Halley / Newton steps ----------------------------------------------------
+  // A walk that is not the last one also writes down the scores above the bracket's lower end (the only ones
+  // later steps can see: tau never drops below it).  They go to the V tile buffers, idle until the output walk:
+  // every wave owns a share of them, cut into chunks of kChunk scores.  A lane keeps its own list -- the ids of
+  // up to eight chunks live in registers -- and draws a chunk from the wave's counter when the last one is full,
+  // so a row with a flat top can take many while most take one.  When no lane of the
+  // block ran out of chunks, the remaining steps run on these lists without touching K again; otherwise the
+  // block keeps walking, as it does when the histogram already shows more candidates than the chunks could hold.
+  constexpr int kChunk = 8;
+  constexpr int kLaneChunks = 8;
+  constexpr bool kTwoV = (G::kNBuf == 2 && !G::kVSingle);
+  constexpr int kWavePoolBytes = kTwoV ? G::kVTile / (NW / 2) : G::kVTile / NW;
+  constexpr int kChunksRaw = kWavePoolBytes / (kChunk * 4);
+  constexpr int kChunks = kChunksRaw > 128 ? 128 : kChunksRaw;  // chunk ids are bytes
+  constexpr bool kLists = kChunks >= 96;                         // one chunk a lane and some to spare
+  float* const my_pool = reinterpret_cast<float*>(
+      (kTwoV && wave >= NW / 2 ? v_lds1 : v_lds0) + (kTwoV ? wave % (NW / 2) : wave) * kWavePoolBytes);
   {
     float t_prev = br.t, f_prev = 0.f;
+    bool list_mode = false;       // uniform over the block
+    bool may_build = cand_est <= 0.5f * (float)(kChunks * kChunk);  // uniform over the wave; one attempt only
+    int my_n = 0;                      // this lane's list: its length,
+    unsigned long long my_ids = 0ull;  // the ids of its chunks (a byte each, in drawing order),
+    uint32_t my_chunk = 0u;            // the chunk being filled
+    const bool live_row = qi < L;
     for (int it = 0; it < p.niter; ++it) {
+      constexpr bool kWithLists = kMulti && kLists;
       const float init = -br.t * inv_qs;
       const float dl = (br.lo - br.t) * inv_qs;  // z > lo  <=>  (s - t_raw) > dl
-      const bool refine = true;  // every step tightens the tile mask to {z > lower bound} for the next pass
       float a0 = 0.f, a1 = 0.f, a2 = 0.f;
       int cnt_pos = 0, cnt_neg = 0, n_seen = 0;  // n_seen - cnt_neg: scores above the threshold (packed path)
+      // one score's terms in fp32; r = raw score - raw threshold
+      auto add_score = [&](float r) {
+        if constexpr (AM == ATT_15) {
+          const float u = __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
+          a0 = fmaf(u, u, a0);
+          a1 += u;
+          cnt_pos += r > 0.f;
+        } else if constexpr (AM == ATT_2) {
+          a0 += __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
+          cnt_pos += r > 0.f;
+        } else {
+          if (r > 0.f) {
+            const float uz = r * qs;
+            const float e0 = fast_exp2(fast_log2(uz) * p.c0);
+            const float rc = fast_rcp(uz);
+            const float e1 = e0 * rc;
+            a0 += e0;
+            a1 += e1;
+            a2 += e1 * rc;
+          }
+        }
+      };
+      bool build = kWithLists && !list_mode && may_build && it + 1 < p.niter;  // uniform over the wave
+      bool lane_full = false;
+      const bool collecting = build;
+      // the lane's candidates of a block join its list; the wave stops collecting once a lane is out of room
+      auto append_block = [&](const f32x16& sc) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          if (sc[i] > dl && live_row && !lane_full) {
+            if (my_n % kChunk == 0) {
+              const uint32_t c = my_n < kChunk * kLaneChunks ? atomicAdd(&chunk_ctr[wave], 1u) : (uint32_t)kChunks;
+              if (c < (uint32_t)kChunks) {
+                my_chunk = c;
+                my_ids |= (unsigned long long)c << my_n;  // byte my_n / 8
+              } else {
+                lane_full = true;
+              }
+            }
+            if (!lane_full) {
+              my_pool[my_chunk * kChunk + my_n % kChunk] = sc[i] - init;
+              ++my_n;
+            }
+          }
+        }
+        if (__builtin_amdgcn_ballot_w64(lane_full) != 0ull) build = false;
+      };
+      if (kWithLists && list_mode) {
+        for (int e = 0; __builtin_amdgcn_ballot_w64(e < my_n) != 0ull; ++e)
+          if (e < my_n) add_score(my_pool[(uint32_t)((my_ids >> (e & ~7)) & 0xffull) * kChunk + e % kChunk] + init);
+      } else {
+      if (build) {
+        my_n = 0;
+        my_ids = 0ull;
+        if (lane == 0) chunk_ctr[wave] = 0u;
+      }
+      const uint32_t* fine_cur = fine_of(mask_cur);
       tile_loop(mask_cur, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
-        float dmax = -INFINITY;
+        const uint32_t bits = block_bits(fine_cur, kt);
+        float dmax0 = -INFINITY, dmax1 = -INFINITY;  // per 32-key block
         if constexpr (k16 && AM != ATT_GEN) {
           // 16-bit inputs: the sums run on pairs of scores rounded (towards zero) to f16 -- packed max, two-term
           // dot products with fp32 accumulation, and the sign bits for the support count: 3.5 VALU
           // instructions per score instead of 5.5.  The rounding moves f by a few 1e-4 relative, far inside
           // the 16-bit output tolerance, and keeps {score > lower bound} a superset (negative values round up).
-          h2_t dm2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+          const h2_t ninf2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+          h2_t dm2[2] = {ninf2, ninf2};
           const h2_t zero2 = {(_Float16)0.f, (_Float16)0.f}, one2 = {(_Float16)1.f, (_Float16)1.f};
-          for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
-            n_seen += 32;
+          for_tile_sel(kt, kt_lds, init, bits, [&](const f32x16& sc, int kb) {
+            n_seen += 16;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-              const float ra = j < 8 ? s0[(2 * j) & 15] : s1[(2 * j) & 15];
-              const float rb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
+            for (int j = 0; j < 8; ++j) {
+              const float ra = sc[2 * j];
+              const float rb = sc[2 * j + 1];
               const h2_t h = pkrtz(ra, rb);
-              dm2 = __builtin_elementwise_max(dm2, h);
+              dm2[kb] = __builtin_elementwise_max(dm2[kb], h);
               cnt_neg += __builtin_popcount(__builtin_bit_cast(uint32_t, h) & 0x80008000u);
               const h2_t u = __builtin_elementwise_max(h, zero2);
               if constexpr (AM == ATT_15) {
@@ -752,42 +924,32 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
                 a0 = __builtin_amdgcn_fdot2(u, one2, a0, false);
               }
             }
+            if (build && __builtin_amdgcn_ballot_w64(live_row && fmaxf((float)dm2[kb][0], (float)dm2[kb][1]) > dl) != 0ull) append_block(sc);
           });
-          dmax = fmaxf((float)dm2[0], (float)dm2[1]);
+          dmax0 = fmaxf((float)dm2[0][0], (float)dm2[0][1]);
+          dmax1 = fmaxf((float)dm2[1][0], (float)dm2[1][1]);
         } else {
-        for_tile(kt, kt_lds, init, [&](const f32x16& s0, const f32x16& s1) {
-          if (refine) {
+          for_tile_sel(kt, kt_lds, init, bits, [&](const f32x16& sc, int kb) {
+            float dm = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) dmax = fmaxf(fmaxf(dmax, s0[i]), s1[i]);
-          }
+            for (int i = 0; i < 16; ++i) dm = fmaxf(dm, sc[i]);
+            if (kb == 0) dmax0 = dm;
+            else dmax1 = dm;
 #pragma unroll
-          for (int i = 0; i < 32; ++i) {
-            const float r = i < 16 ? s0[i & 15] : s1[i & 15];
-            if constexpr (AM == ATT_15) {
-              const float u = __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
-              a0 = fmaf(u, u, a0);
-              a1 += u;
-              cnt_pos += r > 0.f;
-            } else if constexpr (AM == ATT_2) {
-              a0 += __builtin_amdgcn_fmed3f(r, 0.f, INFINITY);
-              cnt_pos += r > 0.f;
-            } else {
-              if (r > 0.f) {
-                const float uz = r * qs;
-                const float e0 = fast_exp2(fast_log2(uz) * p.c0);
-                const float rc = fast_rcp(uz);
-                const float e1 = e0 * rc;
-                a0 += e0;
-                a1 += e1;
-                a2 += e1 * rc;
-              }
-            }
-          }
-        });
+            for (int i = 0; i < 16; ++i) add_score(sc[i]);
+            if (build && __builtin_amdgcn_ballot_w64(live_row && dm > dl) != 0ull) append_block(sc);
+          });
         }
-        if (refine && __builtin_amdgcn_ballot_w64(dmax > dl) != 0ull && lane == 0) mark_tile(mask_new, kt);
+        // every step tightens the masks to {z > lower bound} for the next walk
+        if constexpr (kFine) {
+          const uint32_t nb = (__builtin_amdgcn_ballot_w64(dmax0 > dl) != 0ull ? 1u : 0u) | (__builtin_amdgcn_ballot_w64(dmax1 > dl) != 0ull ? 2u : 0u);
+          if (nb && lane == 0) mark_blocks(mask_new, fine_new, kt, nb);
+        } else {
+          if (__builtin_amdgcn_ballot_w64(fmaxf(dmax0, dmax1) > dl) != 0ull && lane == 0) mark_tile(mask_new, kt);
+        }
       });
       if constexpr (k16 && AM != ATT_GEN) cnt_pos = n_seen - cnt_neg;
+      }
       if constexpr (AM == ATT_15) {
         a0 *= qs * qs;
         a1 *= qs;
@@ -804,12 +966,24 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       // for this row and the unconditional bound takes its place.
       if (a0 > 1.f && br.t + (a0 - 1.f) / (p.c0 * a1) > br.hi) br.hi = hi_cap;
       hybrid_step(br, a0, a1, a2, p.c0, AM != ATT_2 && p.alpha <= 1.5f, p.alpha <= 2.0f, it > 0, t_prev, f_prev);
-      if (refine) {
+      if (!(kWithLists && list_mode)) {
+        if (kWithLists && it + 1 < p.niter) {
+          // a wave that gave up, or did not try, keeps the whole block walking
+          const bool ovf = !collecting || !build;
+          if (ovf && lane == 0) list_flag[it & 1] = 1u;
+          // the other flag word is the next step's; its last readers passed this walk's barriers already
+          if (tid == 0) list_flag[(it + 1) & 1] = 0u;
+        }
         // the mask just written becomes the one to read; the other array is cleared for a later pass
         __syncthreads();
         mask_cur = mask_new;
         mask_new = (mask_cur == mask_a) ? mask_b : mask_a;
-        for (int i = tid; i < p.mask_words; i += G::kThreads) mask_new[i] = 0u;
+        fine_new = fine_of(mask_new);
+        clear_mask(mask_new);
+        if (kWithLists && it + 1 < p.niter) {
+          if (list_flag[it & 1] == 0u) list_mode = true;
+          else may_build = false;
+        }
       }
     }
   }
@@ -829,7 +1003,9 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   unsigned active16 = 0;  // 16x16 score tiles with a non-zero probability (wave-uniform count)
   {
     const float init = -tau * inv_qs;
+    const uint32_t* fine_cur = fine_of(mask_cur);
     tile_loop(mask_cur, true, [&](int kt, const unsigned char* kt_lds, const unsigned char* vt_lds) {
+      const uint32_t bits = block_bits(fine_cur, kt);
       bool tile_active = false;
       // single V tile: every wave joins one barrier per tile once its own share of V has landed (the K loads of
       // the next tile, issued after it, may still be in flight), whether or not it has work in the tile
@@ -844,7 +1020,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           }
         }
       };
-      for_tile_blocks(kt, kt_lds, init, [&](const f32x16& acc, int kb) {
+      for_tile_blocks(kt, kt_lds, init, bits, [&](const f32x16& acc, int kb) {
         float pv[16];
         float hsum[2] = {0.f, 0.f};  // over the lane's keys of each 16-key half of the block
 #pragma unroll

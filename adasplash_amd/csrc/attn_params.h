@@ -25,6 +25,7 @@ struct AttnParams {
   int B, Hq, Hkv, N, Npad;
   int n_mblk;      // 128-row blocks per (b, h) in bmask
   int mask_words;  // int32 words per row block in bmask
+  int fine_masks;  // set by the launch: the kernel keeps per-wave 32-key block bits beside the tile masks
   int niter;
   int causal;
   int use_hist;

@@ -114,3 +114,73 @@ def test_full_size_block_mask_workload_sampled_rows():
         rows = [0, 127, 128, 8191, 16383]
         want = oracle_rows_of_attention(q, k, v, b, h, rows, 1.333, False, N)
         assert max_err(out[b, h, rows], want) < 2e-2
+
+
+# ---- several solver steps: the steps after a walk run on per-lane candidate lists when those fit -------------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("alpha", [1.333, 1.5, 2.0])
+@pytest.mark.parametrize("D,causal,scale", [(64, False, 2.0), (128, True, 2.0), (32, False, 2.0)])
+def test_many_steps_on_peaked_scores(dtype, alpha, D, causal, scale):
+    # few scores within 1 of a row's maximum: every block solves on its lists after the first walk
+    g = torch.Generator().manual_seed(7)
+    B, H, N = 2, 2, 1024
+    q = (scale * torch.randn(B, H, N, D, generator=g)).to(dtype)
+    k = (scale * torch.randn(B, H, N, D, generator=g)).to(dtype)
+    v = torch.randn(B, H, N, D, generator=g).to(dtype)
+    varlen = torch.tensor([N, 700])
+    out = run_v1(q, k, v, alpha=alpha, is_causal=causal, niter=12, varlen=varlen).cpu()
+    want = exact.dense_entmax_attention(q, k, v, alpha, causal, varlen=varlen)
+    assert max_err(out, want) < tol_for(dtype, alpha)
+    assert (out[1, :, 700:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("alpha", [1.333, 1.5])
+def test_flat_rows_beside_peaked_rows(dtype, alpha):
+    # rows whose scores are all equal have as many candidates as keys: their lanes run out of list space and
+    # the block keeps walking, with the same result for the peaked rows that share it
+    g = torch.Generator().manual_seed(11)
+    B, H, N, D = 1, 2, 2048, 64
+    q = (3 * torch.randn(B, H, N, D, generator=g)).to(dtype)
+    k = (3 * torch.randn(B, H, N, D, generator=g)).to(dtype)
+    v = torch.randn(B, H, N, D, generator=g).to(dtype)
+    flat = [5, 130, 131, 1000]
+    q[:, :, flat] = 0
+    out = run_v1(q, k, v, alpha=alpha, is_causal=False, niter=10).cpu()
+    want = exact.dense_entmax_attention(q, k, v, alpha, False)
+    assert max_err(out, want) < tol_for(dtype, alpha)
+    mean_v = v.double().mean(2, keepdim=True)
+    assert max_err(out[:, :, flat], mean_v.expand(-1, -1, len(flat), -1)) < tol_for(dtype, alpha)
+
+
+@pytest.mark.parametrize("n_top", [9, 24, 40, 70, 200])
+def test_rows_with_a_wide_top(n_top):
+    # n_top keys tie for the maximum of every row: past 8 a lane draws further chunks, past 64 per lane (or when
+    # the wave's chunks run out) the block falls back to walking
+    g = torch.Generator().manual_seed(13)
+    B, H, N, D = 1, 1, 1024, 64
+    k = torch.zeros(B, H, N, D)
+    k[..., 0] = -4.0
+    k[:, :, :n_top, 0] = 4.0
+    k[..., 1:] = 0.05 * torch.randn(B, H, N, D - 1, generator=g)
+    q = torch.zeros(B, H, N, D)
+    q[..., 0] = 8.0
+    v = torch.randn(B, H, N, D, generator=g)
+    for alpha in (1.5, 1.333):
+        out = run_v1(q, k, v, alpha=alpha, is_causal=False, niter=10).cpu()
+        want = exact.dense_entmax_attention(q, k, v, alpha, False)
+        assert max_err(out, want) < tol_for(torch.float32, alpha)
+
+
+def test_many_steps_match_between_versions():
+    # adasplash_v2 with several steps takes the same list path behind the histogram
+    g = torch.Generator().manual_seed(17)
+    q = (3 * torch.randn(1, 4, 2048, 128, generator=g)).to(torch.bfloat16)
+    k = (3 * torch.randn(1, 2, 2048, 128, generator=g)).to(torch.bfloat16)
+    v = torch.randn(1, 2, 2048, 128, generator=g).to(torch.bfloat16)
+    out = A.adasplash_v2(q.to(DEV), k.to(DEV), v.to(DEV), niter=4).cpu()
+    kk, vv = k.repeat_interleave(2, 1), v.repeat_interleave(2, 1)
+    want = exact.dense_entmax_attention(q, kk, vv, 1.5, True)
+    assert max_err(out, want) < 2e-2
