@@ -123,8 +123,14 @@ __device__ __forceinline__ void hybrid_step(Bracket& br, float a0, float a1, flo
     has = ok;
   }
   {
-    float tn = t - ff / df;
-    bool ok = allow_newton && !has && tn > lo && tn < hi && fabsf(df) > EPS_DEN;
+    // From the right of the root a Newton step of the convex f can land below the bracket, by a rounding error
+    // when the root is the lower end itself (one entry carries all the mass) or by far when the support grows
+    // quickly to the left.  The root is not down there: the lower end is the best point in that direction, and
+    // from it every later Newton step approaches the root from the left without passing it.
+    // The ends themselves are acceptable (eps is smaller than the spacing of floats at large scores, so a strict
+    // test would turn the exact landing on the lower end into an endless bisection towards it).
+    float tn = fmaxf(t - ff / df, br.lo);
+    bool ok = allow_newton && !has && tn >= lo && tn <= hi && fabsf(df) > EPS_DEN;
     cand = ok ? tn : cand;
     has = has || ok;
   }
