@@ -143,6 +143,9 @@ __device__ __forceinline__ float solve_row(const Row& row, const RowsParams& p, 
     row_sum<TPR, 3>(a, sm);
     if (it >= p.n_iter && fabsf(a[0] - 1.f) <= 2e-6f) break;
     hybrid_step(br, a[0], a[1], a[2], p.c0, p.allow_halley, p.allow_newton, it > 0, t_prev, f_prev);
+    // at large |tau| the spacing of floats keeps |f| above any fixed bound (alpha = 2, inputs of size 16:
+    // f moves in steps of 2e-6 per support entry); a step that no longer moves tau ends the search as well
+    if (it >= p.n_iter && fabsf(br.t - t) <= 2.4e-7f * fabsf(t)) break;
   }
   return br.t;
 }
