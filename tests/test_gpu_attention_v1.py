@@ -199,3 +199,18 @@ def test_one_dominant_key_converges_in_a_few_steps(alpha):
     out = run_v1(q, k, v, alpha=alpha, is_causal=False, niter=5).cpu()
     want = exact.dense_entmax_attention(q, k, v, alpha, False)
     assert max_err(out, want) < 1e-4
+
+
+def test_many_steps_beyond_the_block_bit_limit():
+    # past 128K keys the multi-step kernel keeps only the tile masks (no per-wave block bits); the candidate
+    # lists still serve the later steps
+    g = torch.Generator().manual_seed(23)
+    B, H, N, D = 1, 1, 131072 + 2048, 64
+    q = (3 * torch.randn(B, H, N, D, generator=g)).to(torch.bfloat16)
+    k = (3 * torch.randn(B, H, N, D, generator=g)).to(torch.bfloat16)
+    v = torch.randn(B, H, N, D, generator=g).to(torch.bfloat16)
+    out = run_v1(q, k, v, alpha=1.5, is_causal=True, niter=6, varlen=torch.tensor([N])).cpu()
+    assert torch.isfinite(out.float()).all()
+    rows = [0, 63, 4097, 70000, N - 1]
+    want = oracle_rows_of_attention(q, k, v, 0, 0, rows, 1.5, True, N)
+    assert max_err(out[0, 0, rows], want) < 2e-2
