@@ -31,7 +31,7 @@ FLAGS = [
 # The attention kernels never produce or consume NaNs on purpose (masked scores are -inf and are clamped
 # before any product), so fmax/fmin need no sNaN-quieting pre-pass there.
 _ATTN_FLAGS = ["-fno-honor-nans"] + os.environ.get("ADSP_ATTN_FLAGS", "").split()
-EXTRA_FLAGS = {"attn_bf16": _ATTN_FLAGS, "attn_f16": _ATTN_FLAGS, "attn_f32": _ATTN_FLAGS}
+EXTRA_FLAGS = {f"attn_{kind}{ty}": _ATTN_FLAGS for kind in ("", "multi_") for ty in ("bf16", "f16", "f32")}
 
 
 def _compile(src: Path) -> Path:
