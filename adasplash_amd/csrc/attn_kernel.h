@@ -811,28 +811,33 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   // ---- pass C: niter safeguarded Halley / Newton steps ----------------------------------------------------
   // A walk that is not the last one also writes down the scores above the bracket's lower end (the only ones
   // later steps can see: tau never drops below it).  They go to the V tile buffers, idle until the output walk:
-  // every wave owns a share of them, cut into chunks of kChunk scores.  A lane keeps its own list -- the ids of
-  // up to eight chunks live in registers -- and draws a chunk from the wave's counter when the last one is full,
-  // so a row with a flat top can take many while most take one.  When no lane of the
-  // block ran out of chunks, the remaining steps run on these lists without touching K again; otherwise the
-  // block keeps walking, as it does when the histogram already shows more candidates than the chunks could hold.
-  constexpr int kChunk = 8;
+  // every wave owns a share of them, cut into chunks of kChunk (score, key index) pairs.  A lane keeps its own
+  // list -- the ids of up to eight chunks live in registers -- and draws a chunk from the wave's counter when the
+  // last one is full, so a row with a flat top can take many while most take one.  When no lane of the block ran
+  // out of chunks, the remaining steps run on these lists without touching K again, and so does the output (the
+  // V rows of the listed keys are gathered); otherwise the block keeps walking, as it does when the histogram
+  // already shows more candidates than the chunks could hold.
+  constexpr int kChunk = 4;       // entries per chunk: four scores, then their four key indices
   constexpr int kLaneChunks = 8;
   constexpr bool kTwoV = (G::kNBuf == 2 && !G::kVSingle);
   constexpr int kWavePoolBytes = kTwoV ? G::kVTile / (NW / 2) : G::kVTile / NW;
-  constexpr int kChunksRaw = kWavePoolBytes / (kChunk * 4);
+  constexpr int kChunksRaw = kWavePoolBytes / (kChunk * 8);
   constexpr int kChunks = kChunksRaw > 128 ? 128 : kChunksRaw;  // chunk ids are bytes
   constexpr bool kLists = kChunks >= 96;                         // one chunk a lane and some to spare
   float* const my_pool = reinterpret_cast<float*>(
       (kTwoV && wave >= NW / 2 ? v_lds1 : v_lds0) + (kTwoV ? wave % (NW / 2) : wave) * kWavePoolBytes);
+  bool list_mode = false;            // uniform over the block
+  int my_n = 0;                      // this lane's list: its length,
+  unsigned long long my_ids = 0ull;  // the ids of its chunks (a byte each, in drawing order)
+  const bool live_row = qi < L;
+  // entry e of the lane's list: the score and the key index sit kChunk words apart
+  auto list_slot = [&](int e) -> float* {
+    return my_pool + (uint32_t)((my_ids >> (8 * (e / kChunk))) & 0xffull) * (2 * kChunk) + e % kChunk;
+  };
   {
     float t_prev = br.t, f_prev = 0.f;
-    bool list_mode = false;       // uniform over the block
     bool may_build = cand_est <= 0.5f * (float)(kChunks * kChunk);  // uniform over the wave; one attempt only
-    int my_n = 0;                      // this lane's list: its length,
-    unsigned long long my_ids = 0ull;  // the ids of its chunks (a byte each, in drawing order),
     uint32_t my_chunk = 0u;            // the chunk being filled
-    const bool live_row = qi < L;
     for (int it = 0; it < p.niter; ++it) {
       constexpr bool kWithLists = kMulti && kLists;
       const float init = -br.t * inv_qs;
@@ -865,7 +870,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       bool lane_full = false;
       const bool collecting = build;
       // the lane's candidates of a block join its list; the wave stops collecting once a lane is out of room
-      auto append_block = [&](const f32x16& sc) {
+      auto append_block = [&](const f32x16& sc, int key0) {  // key0: the lane's first key of the block
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           if (sc[i] > dl && live_row && !lane_full) {
@@ -873,13 +878,15 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
               const uint32_t c = my_n < kChunk * kLaneChunks ? atomicAdd(&chunk_ctr[wave], 1u) : (uint32_t)kChunks;
               if (c < (uint32_t)kChunks) {
                 my_chunk = c;
-                my_ids |= (unsigned long long)c << my_n;  // byte my_n / 8
+                my_ids |= (unsigned long long)c << (8 * (my_n / kChunk));
               } else {
                 lane_full = true;
               }
             }
             if (!lane_full) {
-              my_pool[my_chunk * kChunk + my_n % kChunk] = sc[i] - init;
+              float* slot = my_pool + my_chunk * (2 * kChunk) + my_n % kChunk;
+              slot[0] = sc[i] - init;
+              slot[kChunk] = __builtin_bit_cast(float, (uint32_t)(key0 + 8 * (i >> 2) + (i & 3)));
               ++my_n;
             }
           }
@@ -888,7 +895,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       };
       if (kWithLists && list_mode) {
         for (int e = 0; __builtin_amdgcn_ballot_w64(e < my_n) != 0ull; ++e)
-          if (e < my_n) add_score(my_pool[(uint32_t)((my_ids >> (e & ~7)) & 0xffull) * kChunk + e % kChunk] + init);
+          if (e < my_n) add_score(*list_slot(e) + init);
       } else {
       if (build) {
         my_n = 0;
@@ -924,7 +931,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
                 a0 = __builtin_amdgcn_fdot2(u, one2, a0, false);
               }
             }
-            if (build && __builtin_amdgcn_ballot_w64(live_row && fmaxf((float)dm2[kb][0], (float)dm2[kb][1]) > dl) != 0ull) append_block(sc);
+            if (build && __builtin_amdgcn_ballot_w64(live_row && fmaxf((float)dm2[kb][0], (float)dm2[kb][1]) > dl) != 0ull) append_block(sc, kt * kBN + kb * 32 + 4 * lh);
           });
           dmax0 = fmaxf((float)dm2[0][0], (float)dm2[0][1]);
           dmax1 = fmaxf((float)dm2[1][0], (float)dm2[1][1]);
@@ -937,7 +944,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
             else dmax1 = dm;
 #pragma unroll
             for (int i = 0; i < 16; ++i) add_score(sc[i]);
-            if (build && __builtin_amdgcn_ballot_w64(live_row && dm > dl) != 0ull) append_block(sc);
+            if (build && __builtin_amdgcn_ballot_w64(live_row && dm > dl) != 0ull) append_block(sc, kt * kBN + kb * 32 + 4 * lh);
           });
         }
         // every step tightens the masks to {z > lower bound} for the next walk
@@ -1001,7 +1008,76 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float psum = 0.f;
   unsigned active16 = 0;  // 16x16 score tiles with a non-zero probability (wave-uniform count)
-  {
+  // With the lists in place (and no tile statistics asked for) there is nothing to walk: a lane turns its
+  // listed scores into probabilities and adds up the V rows of their keys, read from the row-major V.
+  const bool gather = kMulti && kLists && list_mode && !p.tile_counts;
+  if (gather) {
+    if constexpr (kMulti && kLists) {
+      const float init = -tau * inv_qs;
+      constexpr int kDP = D < 64 ? D : 64;  // output columns per sweep over the list
+      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kEB;
+#pragma unroll 1
+      for (int d0 = 0; d0 < D; d0 += kDP) {
+        float acc[kDP];
+#pragma unroll
+        for (int d = 0; d < kDP; ++d) acc[d] = 0.f;
+        for (int e = 0; __builtin_amdgcn_ballot_w64(e < my_n) != 0ull; ++e) {
+          if (e < my_n) {
+            const float* slot = list_slot(e);
+            const float pv = attn_prob<AM>(slot[0] + init, qs, p.c0);
+            if (pv > 0.f) {
+              const uint32_t key = __builtin_bit_cast(uint32_t, slot[kChunk]);
+              if (d0 == 0) {
+                psum += pv;
+                if (bmask_out) mark_tile(mask_out0 + half * p.mask_words, (int)(key / kBN));
+              }
+              const u32x4* vr = reinterpret_cast<const u32x4*>(vrows + ((size_t)key * D + d0) * G::kEB);
+              if constexpr (k16) {
+#pragma unroll
+                for (int c = 0; c < kDP / 8; ++c) {
+                  const u32x4 w = vr[c];
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) {
+                    const uint32_t ww = w[j];
+                    acc[8 * c + 2 * j] = fmaf(pv, unpack_lo<T>(ww), acc[8 * c + 2 * j]);
+                    acc[8 * c + 2 * j + 1] = fmaf(pv, unpack_hi<T>(ww), acc[8 * c + 2 * j + 1]);
+                  }
+                }
+              } else {
+#pragma unroll
+                for (int c = 0; c < kDP / 4; ++c) {
+                  const u32x4 w = vr[c];
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) {
+                    const uint32_t ww = w[j];
+                    acc[4 * c + j] = fmaf(pv, __builtin_bit_cast(float, ww), acc[4 * c + j]);
+                  }
+                }
+              }
+            }
+          }
+        }
+        // the two lanes of a row each hold half of its output columns (8 g + 4 lh + j of every 32): a lane
+        // keeps its half of its own sums and receives the partner's sums for that half
+#pragma unroll
+        for (int dbl = 0; dbl < kDP / 32; ++dbl) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float lo_part = acc[dbl * 32 + 8 * g + j], hi_part = acc[dbl * 32 + 8 * g + 4 + j];
+              const float own = lh ? hi_part : lo_part, send = lh ? lo_part : hi_part;
+              const float sum = own + __shfl_xor(send, 32, 64);
+              // (the sweep index is a run-time value: select the accumulator instead of indexing it)
+#pragma unroll
+              for (int db = 0; db < G::kDB; ++db)
+                if (db == d0 / 32 + dbl) o[db][4 * g + j] = sum;
+            }
+          }
+        }
+      }
+    }
+  } else {
     const float init = -tau * inv_qs;
     const uint32_t* fine_cur = fine_of(mask_cur);
     tile_loop(mask_cur, true, [&](int kt, const unsigned char* kt_lds, const unsigned char* vt_lds) {

@@ -38,11 +38,11 @@ def run_case(alpha, causal, B, Hq, Hkv, N, D, dtype, varlen=None, version=1, see
     return (qg.grad, kg.grad, vg.grad), want
 
 
-def check(got, want, dtype):
+def check(got, want, dtype, tol_scale=1.0):
     for name, g, w in zip(("dq", "dk", "dv"), got, want):
         assert g.dtype == dtype and g.shape == w.shape
         assert torch.isfinite(g).all(), name
-        assert max_err(g, w) < grad_tol(dtype), name
+        assert max_err(g, w) < tol_scale * grad_tol(dtype), name
 
 
 @pytest.mark.parametrize("N,D", [(128, 64), (256, 128), (512, 32), (128, 16), (128, 256)])
@@ -134,3 +134,14 @@ def test_padding_rows_may_hold_anything(dtype, version, D):
     for a, b in zip(clean, soiled):
         assert torch.isfinite(b).all()
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("version,alpha", [(1, 1.333), (1, 2.0), (2, 1.5)])
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.bfloat16, 128)])
+def test_backward_after_a_forward_on_candidate_lists(version, alpha, dtype, D):
+    # peaked scores: the forward's later solver steps and its output run on the per-lane lists, and the tile mask
+    # the backward consumes comes from the listed keys
+    causal = version == 2
+    got, want = run_case(alpha, causal, 1, 2, 2, 1024, D, dtype, version=version, seed=3, scale=2.0)
+    # dq and dk are linear in k and q, which are twice the size the 16-bit tolerance was set for
+    check(got, want, dtype, tol_scale=1.0 if dtype == torch.float32 else 2.0)

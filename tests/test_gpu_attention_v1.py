@@ -214,3 +214,17 @@ def test_many_steps_beyond_the_block_bit_limit():
     rows = [0, 63, 4097, 70000, N - 1]
     want = oracle_rows_of_attention(q, k, v, 0, 0, rows, 1.5, True, N)
     assert max_err(out[0, 0, rows], want) < 2e-2
+
+
+def test_output_from_lists_matches_output_walk():
+    # asking for tile statistics makes the kernel walk for the output; without them it gathers the V rows of the
+    # listed keys: the same probabilities either way
+    g = torch.Generator().manual_seed(29)
+    q, k = ((3 * torch.randn(2, 2, 2048, 64, generator=g)).to(torch.bfloat16).to(DEV) for _ in range(2))
+    v = torch.randn(2, 2, 2048, 64, generator=g).to(torch.bfloat16).to(DEV)
+    varlen = torch.tensor([2048, 1500]).to(DEV)
+    walked, _, _ = tile_sparsity(q, k, v, alpha=1.333, is_causal=False, niter=10, varlen=varlen)
+    gathered = A.adasplash_v1(q, k, v, alpha=1.333, is_causal=False, niter=10, varlen=varlen)
+    assert max_err(walked.cpu(), gathered.cpu().double()) < 2e-2  # one bf16 step: the walk rounds P to bf16 before its PV product
+    want = exact.dense_entmax_attention(q.cpu(), k.cpu(), v.cpu(), 1.333, False, varlen=varlen.cpu())
+    assert max_err(gathered.cpu(), want) < 2e-2
