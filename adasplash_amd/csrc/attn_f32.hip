@@ -1,8 +1,10 @@
-// attn_fwd_kernel instantiations for element type float: no or one solver step.
+// attn_fwd_kernel instantiations for element type float: no solver step, or one behind the histogram.
 #include "attn_launch.h"
 namespace adsp {
 int launch_attn_multi_f32(const AttnParams& p, int D, int am, hipStream_t s);
 int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s) {
-  return p.niter >= 2 ? launch_attn_multi_f32(p, D, am, s) : launch_attn<float, false>(p, D, am, s);
+  // one step without the histogram is the block-mask variant's: made for sparse supports, which the lists serve
+  const bool multi = p.niter >= 2 || (p.niter == 1 && !p.use_hist);
+  return multi ? launch_attn_multi_f32(p, D, am, s) : launch_attn<float, false>(p, D, am, s);
 }
 }  // namespace adsp

@@ -142,10 +142,18 @@ template <int AM> __device__ __forceinline__ float attn_prob(float r, float qs, 
   return r > 0.f ? fast_exp2(fast_log2(r * qs) * c0) : 0.f;
 }
 
-// kMulti: the instance for two and more solver steps, which carries the candidate lists of the solver walks; the
-// other one (no or one step) does not pay for their registers.
+// Waves per SIMD the kernel is compiled for.  The list-carrying instance does not fit the 168 registers of three
+// waves at 16-bit D = 128 (its solver walk spilled a hundred of them): it gets two waves' worth there.
+template <typename T, int D, bool kMulti> constexpr int fwd_min_waves() {
+  return (kMulti && TileGeo<T, D>::kVSingle) ? 2 : TileGeo<T, D>::kMinWaves;
+}
+
+// kMulti: the instance that carries the candidate lists of the solver walks and the per-wave block bits; it serves
+// two and more solver steps, and a single step without the histogram (the block-mask variant, made for sparse
+// supports).  The other one (no step, or one step behind the histogram) does not pay for their registers.
 template <typename T, int D, int AM, bool kMulti>
-__global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_waves_per_eu(TileGeo<T, D>::kMinWaves, (TileGeo<T, D>::kMinWaves > 2 ? TileGeo<T, D>::kMinWaves : 2)))) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__((TileGeo<T, D>::kThreads))
+__attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves<T, D, kMulti>() > 2 ? fwd_min_waves<T, D, kMulti>() : 2)))) void attn_fwd_kernel(AttnParams p) {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
   using VS = Swz<G::kVRow>;
@@ -866,7 +874,9 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
           }
         }
       };
-      bool build = kWithLists && !list_mode && may_build && it + 1 < p.niter;  // uniform over the wave
+      // lists serve the later steps and, unless tile statistics are asked for, the output
+      const bool want_lists = it + 1 < p.niter || !p.tile_counts;
+      bool build = kWithLists && !list_mode && may_build && want_lists;  // uniform over the wave
       bool lane_full = false;
       const bool collecting = build;
       // the lane's candidates of a block join its list; the wave stops collecting once a lane is out of room
@@ -942,9 +952,12 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
             for (int i = 0; i < 16; ++i) dm = fmaxf(dm, sc[i]);
             if (kb == 0) dmax0 = dm;
             else dmax1 = dm;
+            // a block without a score above the lower end (dl <= 0 up to rounding) has none above the threshold
+            if (__builtin_amdgcn_ballot_w64(dm > fminf(dl, 0.f)) != 0ull) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) add_score(sc[i]);
-            if (build && __builtin_amdgcn_ballot_w64(live_row && dm > dl) != 0ull) append_block(sc, kt * kBN + kb * 32 + 4 * lh);
+              for (int i = 0; i < 16; ++i) add_score(sc[i]);
+              if (build && __builtin_amdgcn_ballot_w64(live_row && dm > dl) != 0ull) append_block(sc, kt * kBN + kb * 32 + 4 * lh);
+            }
           });
         }
         // every step tightens the masks to {z > lower bound} for the next walk
@@ -974,7 +987,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
       if (a0 > 1.f && br.t + (a0 - 1.f) / (p.c0 * a1) > br.hi) br.hi = hi_cap;
       hybrid_step(br, a0, a1, a2, p.c0, AM != ATT_2 && p.alpha <= 1.5f, p.alpha <= 2.0f, it > 0, t_prev, f_prev);
       if (!(kWithLists && list_mode)) {
-        if (kWithLists && it + 1 < p.niter) {
+        if (kWithLists && want_lists) {
           // a wave that gave up, or did not try, keeps the whole block walking
           const bool ovf = !collecting || !build;
           if (ovf && lane == 0) list_flag[it & 1] = 1u;
@@ -987,7 +1000,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
         mask_new = (mask_cur == mask_a) ? mask_b : mask_a;
         fine_new = fine_of(mask_new);
         clear_mask(mask_new);
-        if (kWithLists && it + 1 < p.niter) {
+        if (kWithLists && want_lists) {
           if (list_flag[it & 1] == 0u) list_mode = true;
           else may_build = false;
         }
@@ -1014,27 +1027,28 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
   if (gather) {
     if constexpr (kMulti && kLists) {
       const float init = -tau * inv_qs;
-      constexpr int kDP = D < 64 ? D : 64;  // output columns per sweep over the list
       const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kEB;
-#pragma unroll 1
-      for (int d0 = 0; d0 < D; d0 += kDP) {
-        float acc[kDP];
+      // one sweep over the list per 32 output columns: 32 accumulators at a time keep the kernel within the
+      // registers its walks are compiled for
 #pragma unroll
-        for (int d = 0; d < kDP; ++d) acc[d] = 0.f;
+      for (int db = 0; db < G::kDB; ++db) {
+        float acc[32];
+#pragma unroll
+        for (int d = 0; d < 32; ++d) acc[d] = 0.f;
         for (int e = 0; __builtin_amdgcn_ballot_w64(e < my_n) != 0ull; ++e) {
           if (e < my_n) {
             const float* slot = list_slot(e);
             const float pv = attn_prob<AM>(slot[0] + init, qs, p.c0);
             if (pv > 0.f) {
               const uint32_t key = __builtin_bit_cast(uint32_t, slot[kChunk]);
-              if (d0 == 0) {
+              if (db == 0) {
                 psum += pv;
                 if (bmask_out) mark_tile(mask_out0 + half * p.mask_words, (int)(key / kBN));
               }
-              const u32x4* vr = reinterpret_cast<const u32x4*>(vrows + ((size_t)key * D + d0) * G::kEB);
+              const u32x4* vr = reinterpret_cast<const u32x4*>(vrows + ((size_t)key * D + db * 32) * G::kEB);
               if constexpr (k16) {
 #pragma unroll
-                for (int c = 0; c < kDP / 8; ++c) {
+                for (int c = 0; c < 4; ++c) {
                   const u32x4 w = vr[c];
 #pragma unroll
                   for (int j = 0; j < 4; ++j) {
@@ -1045,7 +1059,7 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
                 }
               } else {
 #pragma unroll
-                for (int c = 0; c < kDP / 4; ++c) {
+                for (int c = 0; c < 8; ++c) {
                   const u32x4 w = vr[c];
 #pragma unroll
                   for (int j = 0; j < 4; ++j) {
@@ -1060,19 +1074,12 @@ __global__ __launch_bounds__((TileGeo<T, D>::kThreads)) __attribute__((amdgpu_wa
         // the two lanes of a row each hold half of its output columns (8 g + 4 lh + j of every 32): a lane
         // keeps its half of its own sums and receives the partner's sums for that half
 #pragma unroll
-        for (int dbl = 0; dbl < kDP / 32; ++dbl) {
+        for (int g = 0; g < 4; ++g) {
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float lo_part = acc[dbl * 32 + 8 * g + j], hi_part = acc[dbl * 32 + 8 * g + 4 + j];
-              const float own = lh ? hi_part : lo_part, send = lh ? lo_part : hi_part;
-              const float sum = own + __shfl_xor(send, 32, 64);
-              // (the sweep index is a run-time value: select the accumulator instead of indexing it)
-#pragma unroll
-              for (int db = 0; db < G::kDB; ++db)
-                if (db == d0 / 32 + dbl) o[db][4 * g + j] = sum;
-            }
+          for (int j = 0; j < 4; ++j) {
+            const float lo_part = acc[8 * g + j], hi_part = acc[8 * g + 4 + j];
+            const float own = lh ? hi_part : lo_part, send = lh ? lo_part : hi_part;
+            o[db][4 * g + j] = own + __shfl_xor(send, 32, 64);
           }
         }
       }

@@ -1,5 +1,5 @@
 // Host-side dispatch of attn_fwd_kernel over (head dim, alpha mode) for one element type and one of the two
-// instances (kMulti: two and more solver steps); each (type, instance) pair is a translation unit of its own.
+// instances (kMulti: the one with candidate lists and block bits); each (type, instance) pair is a translation unit of its own.
 #pragma once
 #include "attn_kernel.h"
 
@@ -12,7 +12,7 @@ template <typename T, int D, int AM, bool kMulti> static int launch_attn_one(con
   const long long n_mblk = (p.N + G::kBM - 1) / G::kBM;
   const long long total = (long long)p.B * p.Hkv * n_mblk * group;
   const long long per_xcd = (total + 7) / 8;
-  // dynamic LDS: the tile masks, and in the instance for two and more solver steps, up to 128K keys, the
+  // dynamic LDS: the tile masks, and in the instance with the candidate lists, up to 128K keys, the
   // per-wave block bits as well (beyond that they would cost occupancy)
   AttnParams q = p;
   q.fine_masks = (kMulti && p.mask_words <= 64) ? 1 : 0;

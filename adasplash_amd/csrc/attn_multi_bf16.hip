@@ -1,4 +1,4 @@
-// attn_fwd_kernel instantiations for element type bf16_t: two and more solver steps.
+// attn_fwd_kernel instantiations for element type bf16_t: two and more solver steps, or one without the histogram.
 #include "attn_launch.h"
 namespace adsp {
 int launch_attn_multi_bf16(const AttnParams& p, int D, int am, hipStream_t s) { return launch_attn<bf16_t, true>(p, D, am, s); }
