@@ -642,13 +642,33 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   float cand_est = 0.f;  // with the histogram: how many scores of this wave's rows may lie above that bound
   constexpr float kBinW = 1.f / (float)kAttnBins;  // bin width in z units
   if (!with_hist) {
+    // the max walk already tells which blocks can matter later: those with an entry within 1 (in z) of the lane's
+    // running maximum, a superset of the entries within 1 of the row maximum
     tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
+      bool any0 = false, any1 = false;
       for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
+        float tm0 = s0[0], tm1 = s1[0];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) m_raw = fmaxf(fmaxf(m_raw, s0[i]), s1[i]);
+        for (int i = 1; i < 16; ++i) {
+          tm0 = fmaxf(tm0, s0[i]);
+          tm1 = fmaxf(tm1, s1[i]);
+        }
+        m_raw = fmaxf(m_raw, fmaxf(tm0, tm1));
+        const float keep = m_raw - inv_qs * 1.0001f - 1e-6f * fabsf(m_raw);  // (margin: rounding of the difference)
+        any0 = tm0 > keep;
+        any1 = tm1 > keep;
       });
+      if constexpr (kFine) {
+        const uint32_t nb = (__builtin_amdgcn_ballot_w64(any0) != 0ull ? 1u : 0u) | (__builtin_amdgcn_ballot_w64(any1) != 0ull ? 2u : 0u);
+        if (nb && lane == 0) mark_blocks(mask_new, fine_new, kt, nb);
+      } else {
+        if (__builtin_amdgcn_ballot_w64(any0 || any1) != 0ull && lane == 0) mark_tile(mask_new, kt);
+      }
     });
     m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+    mask_cur = mask_new;
+    mask_new = mask_b;
+    fine_new = fine_of(mask_new);
   } else {
     // The histogram lives on the absolute grid of bins [g / 8, (g + 1) / 8) of z; the solver needs the nine bins
     // g_top - 8 .. g_top below the bin of the row maximum, which cover [max - 1, max] (everything lower is

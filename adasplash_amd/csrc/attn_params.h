@@ -14,7 +14,7 @@ enum AttnAlphaMode { ATT_15 = 0, ATT_2 = 1, ATT_GEN = 2 };
 struct AttnParams {
   const void* q;
   const void* k;
-  const void* v;   // fp32 path: row-major V; 16-bit path: unused
+  const void* v;   // row-major V: the fp32 path walks it; every path gathers rows of it for the list-based output
   const void* vt;  // 16-bit path: key-major permuted copy of V, [B*Hkv, D, Npad]
   void* out;
   float* taus;
