@@ -267,13 +267,9 @@ __device__ __forceinline__ bool bwd_block_map(int units, int inner, int& unit, i
 // ---------------------------------------------------------------------------------------------------------
 // dQ kernel: one block per (K/V head, query head in its group, row block of 128 queries)
 // ---------------------------------------------------------------------------------------------------------
-#ifndef ADSP_DQ_PLAIN_MAXD
-#define ADSP_DQ_PLAIN_MAXD 128
-#endif
-#ifndef ADSP_DQ_WAVES64
-#define ADSP_DQ_WAVES64 3
-#endif
-template <typename T, int D> constexpr int dq_waves() { return (TileGeo<T, D>::k16 && D <= 64) ? ADSP_DQ_WAVES64 : BwdTiles<T, D>::kMinWaves; }
+constexpr int kDqPlainMaxD = 128;  // largest 16-bit head dim whose unmasked blocks take the predicate-free code
+constexpr int kDqWaves64 = 3;      // waves per SIMD of the dQ kernel at 16-bit D <= 64
+template <typename T, int D> constexpr int dq_waves() { return (TileGeo<T, D>::k16 && D <= 64) ? kDqWaves64 : BwdTiles<T, D>::kMinWaves; }
 
 template <typename T, int D, int AM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T, D>()), (dq_waves<T, D>() > 2 ? dq_waves<T, D>() : 2)))) void attn_bwd_dq_kernel(AttnBwdParams p) {
@@ -389,7 +385,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T
   // one fma per score instead of a compare and two selects more.  The choice is a template argument so that each
   // kind of block is one piece of straight-line code, products included.
   // (only where the second code path fits the register budget: at D = 128 it costs spills and more than it saves)
-  constexpr bool kPlainBlocks = k16 && D <= ADSP_DQ_PLAIN_MAXD;
+  constexpr bool kPlainBlocks = k16 && D <= kDqPlainMaxD;
   auto block_is_plain = [&](int kt, int kb) { return kPlainBlocks && kt * kBN + kb * 32 + 31 <= lim_all; };
   auto block_terms = [&](auto plain_c, int kt, int kb, const unsigned char* ka, const unsigned char* va, float (&r)[16],
                          f32x16& dp) {

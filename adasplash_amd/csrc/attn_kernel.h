@@ -832,10 +832,6 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   }
   br.t = 0.5f * (br.lo + br.hi);
 
-#if defined(ADSP_EXP_STOP) && ADSP_EXP_STOP == 1
-  if (p.taus && qi < L && lh == 0) p.taus[(size_t)(b * p.Hq + h) * N + qi] = br.t + hist_lo;
-  return;
-#endif
   // ---- pass C: niter safeguarded Halley / Newton steps ----------------------------------------------------
   // A walk that is not the last one also writes down the scores above the bracket's lower end (the only ones
   // later steps can see: tau never drops below it).  They go to the V tile buffers, idle until the output walk:
@@ -1029,10 +1025,6 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   }
   const float tau = br.t;
 
-#if defined(ADSP_EXP_STOP) && ADSP_EXP_STOP == 2
-  if (p.taus && qi < L && lh == 0) p.taus[(size_t)(b * p.Hq + h) * N + qi] = br.t;
-  return;
-#endif
   // ---- pass D: out = sum_j p_j v_j / sum_j p_j over the masked tiles --------------------------------------
   f32x16 o[G::kDB];
 #pragma unroll

@@ -491,11 +491,9 @@ template <typename T, int AM> static void launch_fwd(const RowsParams& p, bool a
     // 2^27-element problems: bf16 4096 columns 74 % of HBM peak with a wave per row against 42 %, 8192
     // columns 66 % against 74-77 %).
     const long long c16 = (nvec + 15) / 16;
-#ifndef ADSP_ROWS_C16_MAX
-#define ADSP_ROWS_C16_MAX 8
-#endif
+    constexpr long long kShortRowChunks = 8;
     // Short rows: 16 threads per row, four rows to a wave, so that the per-row solve is shared out.
-    if (c16 <= ADSP_ROWS_C16_MAX) {
+    if (c16 <= kShortRowChunks) {
       if (c16 <= 1) return launch_reg<T, AM, 1, 16>(p, s);
       if (c16 <= 2) return launch_reg<T, AM, 2, 16>(p, s);
       if (c16 <= 4) return launch_reg<T, AM, 4, 16>(p, s);
