@@ -30,7 +30,7 @@ def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_co
     ws_bytes = lib.adsp_attn_workspace_bytes(B, Hkv, N, D, dt)
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
     bits = _varlen_bits(varlen)
-    with torch.cuda.device(q.device):
+    with _lib.device_guard(q.device):
         stream = _lib.current_stream(q.device)
         if version == 2:
             st = lib.adsp_attn_v2_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), taus.data_ptr(),
@@ -70,7 +70,7 @@ def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
     zinv = torch.empty((B, Hq, N), device=q.device, dtype=torch.float32)
     ws_bytes = lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dt)
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
-    with torch.cuda.device(q.device):
+    with _lib.device_guard(q.device):
         st = lib.adsp_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), taus.data_ptr(),
                                _lib.ptr(bmask), _lib.ptr(varlen), _varlen_bits(varlen), dq.data_ptr(), dk.data_ptr(),
                                dv.data_ptr(), delta.data_ptr(), zinv.data_ptr(), B, Hq, Hkv, N, D, dt, float(alpha),

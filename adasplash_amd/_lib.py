@@ -4,6 +4,7 @@ There is no CPU or eager fallback: if the library has not been built, or a tenso
 ROCm device, the call fails.
 """
 
+import contextlib
 import ctypes
 from pathlib import Path
 
@@ -66,6 +67,14 @@ def require_device(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:
             raise RuntimeError("adasplash_amd kernels run on a ROCm device only; got a CPU tensor")
+
+
+def device_guard(device):
+    """Context that makes `device` current for the launch; a no-op when it already is (the common case: entering
+    torch's guard costs the host more than a short kernel lasts)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return contextlib.nullcontext()
+    return torch.cuda.device(device)
 
 
 def current_stream(device) -> int:

@@ -22,7 +22,7 @@ class _EntmaxRows(torch.autograd.Function):
         lib = _lib.load()
         y = torch.empty_like(x)  # the kernel writes every element, zeros included
         rows = x.numel() // size_n if size_n > 0 else 0
-        with torch.cuda.device(x.device):
+        with _lib.device_guard(x.device):
             st = lib.adsp_entmax_rows_fwd(x.data_ptr(), y.data_ptr(), rows, size_n, _lib.dtype_code(x), float(alpha),
                                           int(n_iter), int(bool(use_histogram)), int(bool(fast_math)),
                                           _lib.current_stream(x.device))
@@ -42,7 +42,7 @@ class _EntmaxRows(torch.autograd.Function):
         dx = torch.empty_like(dy)
         rows = y.numel() // size_n if size_n > 0 else 0
         lib = _lib.load()
-        with torch.cuda.device(y.device):
+        with _lib.device_guard(y.device):
             st = lib.adsp_entmax_rows_bwd(y.data_ptr(), dy.data_ptr(), dx.data_ptr(), rows, size_n, _lib.dtype_code(y),
                                           float(ctx.alpha), _lib.current_stream(y.device))
         _lib.check(st, "adsp_entmax_rows_bwd")

@@ -142,8 +142,8 @@ def bench_rows(steps, warmup, device, rows=16384, cols=8192):
     for dt, dname in ((torch.bfloat16, "bf16"), (torch.float32, "f32")):
         nbuf = 4
         xs = [base.roll(i, 0).to(dt).to(device) for i in range(nbuf)]
-        # Outputs are allocated once and the launches go through the C ABI: a launch lasts 0.08-0.18 ms, less than
-        # the Python wrapper's allocation and checks take on the host, which would otherwise be what is timed.
+        # Outputs are allocated once and the launches go through the C ABI, so that the timed region holds kernel
+        # launches only (a launch lasts 0.08-0.18 ms; the Python wrapper adds about 13 us of host time per call).
         # 200 untimed launches first (20-40 ms): the first few milliseconds after an idle period run at lower clocks.
         ys = [torch.empty_like(x) for x in xs]
         nbytes = rows * cols * 2 * xs[0].element_size()
