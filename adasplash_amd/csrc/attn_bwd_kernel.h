@@ -59,27 +59,44 @@ template <typename T, int D> struct BwdTiles {
   // DMA of rows [row0, row0 + 64) of a row-major [N][D] tensor into a swizzled tile.
   static __device__ __forceinline__ void issue_rows(const unsigned char* g, int row0, int N, unsigned char* lds, int wave,
                                                     int lane) {
+    // the address is a wave-uniform base plus a 32-bit lane offset; for a whole tile the offset does not depend on the
+    // tile and the base is formed with scalar instructions
+    if (row0 + kBN <= N) {
+      const unsigned char* base = uniform_ptr(g + (size_t)row0 * G::kKRow);
 #pragma unroll
-    for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
-      const int j = j0 * kNW + wave;
-      if (kLoads % kNW == 0 || j < kLoads) {
-        const int P = j * 64 + lane;
-        const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
-        int gr = row0 + row;
-        gr = gr < N ? gr : N - 1;  // rows past the end are masked by the caller
-        dma16(g + (size_t)gr * G::kKRow + c * 16, lds + j * 1024);
+      for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
+        const int j = j0 * kNW + wave;
+        if (kLoads % kNW == 0 || j < kLoads) {
+          const int P = j * 64 + lane;
+          const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
+          dma16s(base, (uint32_t)(row * G::kKRow + c * 16), lds + j * 1024);
+        }
+      }
+    } else {
+      g = uniform_ptr(g);
+#pragma unroll
+      for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
+        const int j = j0 * kNW + wave;
+        if (kLoads % kNW == 0 || j < kLoads) {
+          const int P = j * 64 + lane;
+          const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
+          int gr = row0 + row;
+          gr = gr < N ? gr : N - 1;  // rows past the end are masked by the caller
+          dma16s(g, (uint32_t)gr * (uint32_t)G::kKRow + (uint32_t)(c * 16), lds + j * 1024);
+        }
       }
     }
   }
   // DMA of one contiguous transposed tile ([D][64], as written by vt_layout_kernel) into a swizzled tile.
   static __device__ __forceinline__ void issue_t(const unsigned char* gtile, unsigned char* lds, int wave, int lane) {
+    gtile = uniform_ptr(gtile);
 #pragma unroll
     for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
       const int j = j0 * kNW + wave;
       if (kLoads % kNW == 0 || j < kLoads) {
         const int P = j * 64 + lane;
         const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
-        dma16(gtile + row * G::kVRow + c * 16, lds + j * 1024);
+        dma16s(gtile, (uint32_t)(row * G::kVRow + c * 16), lds + j * 1024);
       }
     }
   }

@@ -85,6 +85,24 @@ __device__ __forceinline__ void dma16(const void* gsrc, void* lds) {
                : "memory");  // (m0 is a reserved register: the compiler sets it itself before each of its own uses)
 }
 
+// The same with the global address split into a wave-uniform base (a scalar register pair) and a 32-bit byte offset per
+// lane: the tile loops keep the lane offsets in registers and form only the tile's base, with scalar instructions.
+// A pointer the caller knows to be the same in every lane, moved to scalar registers (free when the compiler can see
+// that it is uniform, two v_readfirstlane otherwise).
+__device__ __forceinline__ const unsigned char* uniform_ptr(const void* ptr) {
+  const unsigned long long a = (unsigned long long)(uintptr_t)ptr;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));
+  return reinterpret_cast<const unsigned char*>((uintptr_t)(((unsigned long long)hi << 32) | lo));
+}
+__device__ __forceinline__ void dma16s(const void* gbase, uint32_t off, void* lds) {
+  const uint32_t base = (uint32_t)(uintptr_t)lds;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(off), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(base))
+               : "memory");
+}
+
 // 16-byte LDS read at a byte address held as an integer (plus a constant that lands in the instruction's offset field)
 __device__ __forceinline__ u32x4 lds_read16(uint32_t addr, int imm = 0) {
   return *(const __attribute__((address_space(3))) u32x4*)(addr + imm);
@@ -308,7 +326,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
 #pragma unroll
       for (int j0 = 0; j0 < kKPer; ++j0) {
         const int j = j0 * NW + wave;
-        if (G::kKLoads % NW == 0 || j < G::kKLoads) dma16(base + off[j0], lds + j * 1024);
+        if (G::kKLoads % NW == 0 || j < G::kKLoads) dma16s(base, off[j0], lds + j * 1024);
       }
     } else {
 #pragma unroll
@@ -331,7 +349,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
 #pragma unroll
       for (int j0 = 0; j0 < kVPer; ++j0) {
         const int j = j0 * NW + wave;
-        if (G::kVLoads % NW == 0 || j < G::kVLoads) dma16(base + voff[j0], vb + j * 1024);
+        if (G::kVLoads % NW == 0 || j < G::kVLoads) dma16s(base, voff[j0], vb + j * 1024);
       }
     } else {
       issue_rows(vglob, koff, vb, kt);  // same geometry as K
