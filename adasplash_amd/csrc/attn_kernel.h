@@ -298,16 +298,22 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   // belongs to row P / kC, stored chunk P % kC, i.e. logical chunk (P % kC) ^ sw(row).
   // Byte offsets of this lane's pieces inside a tile do not depend on the tile: they are kept in registers
   // and the DMA address is the tile's (wave-uniform) base plus that offset.
+  // A wave's successive loads of a tile lie NW KB apart and NW * 64 / kC rows further down; when that is a multiple of
+  // the swizzle period (16 rows) the lane's offset of load j0 is that of load 0 plus j0 * NW KB, which goes into the
+  // scalar base: one offset register per tile kind instead of one per load.
   constexpr int kKPer = (G::kKLoads + NW - 1) / NW, kVPer = (G::kVLoads + NW - 1) / NW;
-  uint32_t koff[kKPer], voff[kVPer];
+  constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
+  constexpr bool kVStep = (NW * 64 / VS::kC) % 16 == 0 && (NW * 64) % VS::kC == 0;
+  constexpr int kKOffs = kKStep ? 1 : kKPer, kVOffs = kVStep ? 1 : kVPer;
+  uint32_t koff[kKOffs], voff[kVOffs];
 #pragma unroll
-  for (int j0 = 0; j0 < kKPer; ++j0) {
+  for (int j0 = 0; j0 < kKOffs; ++j0) {
     const int P = (j0 * NW + wave) * 64 + lane;
     const int row = P / KS::kC;
     koff[j0] = (uint32_t)(row * G::kKRow + (((P % KS::kC) ^ KS::sw(row)) << 4));
   }
 #pragma unroll
-  for (int j0 = 0; j0 < kVPer; ++j0) {
+  for (int j0 = 0; j0 < kVOffs; ++j0) {
     const int P = (j0 * NW + wave) * 64 + lane;
     const int row = P / VS::kC;
     voff[j0] = (uint32_t)(row * G::kVRow + (((P % VS::kC) ^ VS::sw(row)) << 4));
@@ -319,14 +325,17 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   // c = 4 kb + 2 s + lh.
   const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
   const uint32_t v_lane = (uint32_t)(lq * G::kVRow + ((lh ^ VS::sw(lq)) << 4));
-  auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKPer], unsigned char* lds, int kt) {
+  auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKOffs], unsigned char* lds, int kt) {
     // a row-major [64][D] tile out of a row-major tensor (K, or V for fp32); the last tile may stick out
     const unsigned char* base = g + (size_t)kt * G::kKTile;
     if ((kt + 1) * kBN <= N) {  // one branch per tile, then straight-line loads
 #pragma unroll
       for (int j0 = 0; j0 < kKPer; ++j0) {
         const int j = j0 * NW + wave;
-        if (G::kKLoads % NW == 0 || j < G::kKLoads) dma16s(base, off[j0], lds + j * 1024);
+        if (G::kKLoads % NW == 0 || j < G::kKLoads) {
+          if constexpr (kKStep) dma16s(base + j0 * (NW * 1024), off[0], lds + j * 1024);
+          else dma16s(base, off[j0], lds + j * 1024);
+        }
       }
     } else {
 #pragma unroll
@@ -349,7 +358,10 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
 #pragma unroll
       for (int j0 = 0; j0 < kVPer; ++j0) {
         const int j = j0 * NW + wave;
-        if (G::kVLoads % NW == 0 || j < G::kVLoads) dma16s(base, voff[j0], vb + j * 1024);
+        if (G::kVLoads % NW == 0 || j < G::kVLoads) {
+          if constexpr (kVStep) dma16s(base + j0 * (NW * 1024), voff[0], vb + j * 1024);
+          else dma16s(base, voff[j0], vb + j * 1024);
+        }
       }
     } else {
       issue_rows(vglob, koff, vb, kt);  // same geometry as K
