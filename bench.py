@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these
 # same workloads, each counter scaled by what it reads for a plain 1 GiB copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
-MEASURED_HBM_TRAFFIC_BYTES = {"c4": 1.589e9, "c3": 0.1998e9, "c5": 0.632e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5373e9,
+MEASURED_HBM_TRAFFIC_BYTES = {"c4": 1.511e9, "c3": 0.1998e9, "c5": 0.632e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5373e9,
                               "c2_bwd_f32": 1.0848e9, "c2_bwd_bf16": 0.5476e9,
                               "c4_bwd": 23.57e9}  # c4_bwd: dq kernel 2.03e9 + dk/dv kernel 21.54e9
 
