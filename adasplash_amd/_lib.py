@@ -20,6 +20,7 @@ _vp, _i, _i64, _sz, _dbl = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes
 
 _SIGNATURES = {
     "adsp_version": (_i, []),
+    "adsp_build_id": (ctypes.c_char_p, []),
     "adsp_status_string": (ctypes.c_char_p, [_i]),
     "adsp_entmax_rows_fwd": (_i, [_vp, _vp, _i64, _i64, _i, _dbl, _i, _i, _i, _vp]),
     "adsp_entmax_rows_bwd": (_i, [_vp, _vp, _vp, _i64, _i64, _i, _dbl, _vp]),
@@ -52,8 +53,29 @@ def load():
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
+        _check_build_id(lib)
         _lib = lib
     return _lib
+
+
+def build_id() -> str:
+    """The source hash baked into the loaded library."""
+    return load().adsp_build_id().decode()
+
+
+def _check_build_id(lib):
+    """Refuse a library that was built from other sources than the ones next to it.  The kernel sources travel
+    with the package; when they are absent (a stripped install) there is nothing to compare with."""
+    from . import build as _build
+
+    if not _build.CSRC.is_dir() or not _build.INCLUDE.is_dir():
+        return
+    have, want = lib.adsp_build_id().decode(), _build.source_id()
+    if have != want:
+        raise RuntimeError(
+            f"{_LIB_PATH} is stale: it was built from sources with id {have}, the tree has id {want}. "
+            "Rebuild with `python -m adasplash_amd.build`."
+        )
 
 
 def dtype_code(t: torch.Tensor) -> int:

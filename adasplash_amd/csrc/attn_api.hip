@@ -6,12 +6,26 @@
 #include "../../include/adasplash_hip.h"
 
 namespace adsp {
-int launch_attn_bf16(const AttnParams& p, int D, int am, hipStream_t s);
-int launch_attn_f16(const AttnParams& p, int D, int am, hipStream_t s);
-int launch_attn_f32(const AttnParams& p, int D, int am, hipStream_t s);
-int launch_attn_bwd_bf16(const AttnBwdParams& p, int D, int am, hipStream_t s);
-int launch_attn_bwd_f16(const AttnBwdParams& p, int D, int am, hipStream_t s);
-int launch_attn_bwd_f32(const AttnBwdParams& p, int D, int am, hipStream_t s);
+// The kernels live in one translation unit per (element type, head dim, instance): attn_fwd_unit.hip and
+// attn_bwd_unit.hip, compiled once per combination.
+#define ADSP_DECL_D(tag, d)                                                      \
+  int launch_attn_fwd_##tag##_d##d##_m0(const AttnParams&, int, hipStream_t);   \
+  int launch_attn_fwd_##tag##_d##d##_m1(const AttnParams&, int, hipStream_t);   \
+  int launch_attn_bwd_##tag##_d##d(const AttnBwdParams&, int, hipStream_t);
+#define ADSP_DECL_TAG(tag) ADSP_DECL_D(tag, 16) ADSP_DECL_D(tag, 32) ADSP_DECL_D(tag, 64) ADSP_DECL_D(tag, 128) ADSP_DECL_D(tag, 256)
+ADSP_DECL_TAG(f32)
+ADSP_DECL_TAG(bf16)
+ADSP_DECL_TAG(f16)
+
+typedef int (*attn_fwd_fn)(const AttnParams&, int, hipStream_t);
+typedef int (*attn_bwd_fn)(const AttnBwdParams&, int, hipStream_t);
+#define ADSP_FWD_ROW(tag, d) {launch_attn_fwd_##tag##_d##d##_m0, launch_attn_fwd_##tag##_d##d##_m1}
+#define ADSP_FWD_TAG(tag) {ADSP_FWD_ROW(tag, 16), ADSP_FWD_ROW(tag, 32), ADSP_FWD_ROW(tag, 64), ADSP_FWD_ROW(tag, 128), ADSP_FWD_ROW(tag, 256)}
+#define ADSP_BWD_TAG(tag) {launch_attn_bwd_##tag##_d16, launch_attn_bwd_##tag##_d32, launch_attn_bwd_##tag##_d64, launch_attn_bwd_##tag##_d128, launch_attn_bwd_##tag##_d256}
+// indexed by adsp_dtype (ADSP_F32 = 0, ADSP_BF16 = 1, ADSP_F16 = 2), head dim slot, instance
+static const attn_fwd_fn kFwdTable[3][5][2] = {ADSP_FWD_TAG(f32), ADSP_FWD_TAG(bf16), ADSP_FWD_TAG(f16)};
+static const attn_bwd_fn kBwdTable[3][5] = {ADSP_BWD_TAG(f32), ADSP_BWD_TAG(bf16), ADSP_BWD_TAG(f16)};
+static int head_dim_slot(int D) { return D == 16 ? 0 : (D == 32 ? 1 : (D == 64 ? 2 : (D == 128 ? 3 : (D == 256 ? 4 : -1)))); }
 
 // Tile-wise key-major, MFMA-ordered copy of V for the 16-bit path.  Keys are cut in tiles of 64; a tile
 // is stored as one contiguous [D][64] block (so the kernel fetches it with contiguous kilobyte copies):
@@ -116,8 +130,10 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
     hipLaunchKernelGGL(vt_layout_kernel, dim3(vt_layout_blocks(p.Npad, D), (unsigned)(B * Hkv)), dim3(256), 0, s,
                        (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv);
   }
-  int rc = dtype == ADSP_BF16 ? launch_attn_bf16(p, D, am, s)
-                              : (dtype == ADSP_F16 ? launch_attn_f16(p, D, am, s) : launch_attn_f32(p, D, am, s));
+  // The list-carrying instance serves two and more solver steps, and a single step without the histogram (the
+  // block-mask variant's, made for sparse supports); the other one no step, or one behind the histogram.
+  const bool multi = niter >= 2 || (niter == 1 && !use_hist);
+  int rc = kFwdTable[dtype][head_dim_slot(D)][multi ? 1 : 0](p, am, s);
   if (rc != 0) return ADSP_ERR_LAUNCH;
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
 }
@@ -216,13 +232,17 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     p.qt = qt;
     p.dot = dot;
   }
-  int rc = dtype == ADSP_BF16 ? launch_attn_bwd_bf16(p, D, am, s)
-                              : (dtype == ADSP_F16 ? launch_attn_bwd_f16(p, D, am, s) : launch_attn_bwd_f32(p, D, am, s));
+  int rc = kBwdTable[dtype][head_dim_slot(D)](p, am, s);
   if (rc != 0) return ADSP_ERR_LAUNCH;
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
 }
 
-extern "C" int adsp_version(void) { return 1; }
+extern "C" int adsp_version(void) { return 2; }
+
+#ifndef ADSP_BUILD_ID
+#define ADSP_BUILD_ID "unknown"
+#endif
+extern "C" const char* adsp_build_id(void) { return ADSP_BUILD_ID; }
 
 extern "C" const char* adsp_status_string(int status) {
   switch (status) {

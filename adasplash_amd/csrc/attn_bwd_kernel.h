@@ -821,15 +821,4 @@ template <typename T, int D> static int launch_attn_bwd_d(const AttnBwdParams& p
   return 0;
 }
 
-template <typename T> static int launch_attn_bwd(const AttnBwdParams& p, int D, int am, hipStream_t s) {
-  switch (D) {
-    case 16: return launch_attn_bwd_d<T, 16>(p, am, s);
-    case 32: return launch_attn_bwd_d<T, 32>(p, am, s);
-    case 64: return launch_attn_bwd_d<T, 64>(p, am, s);
-    case 128: return launch_attn_bwd_d<T, 128>(p, am, s);
-    case 256: return launch_attn_bwd_d<T, 256>(p, am, s);
-  }
-  return 2;
-}
-
 }  // namespace adsp

@@ -327,7 +327,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   const uint32_t v_lane = (uint32_t)(lq * G::kVRow + ((lh ^ VS::sw(lq)) << 4));
   auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKOffs], unsigned char* lds, int kt) {
     // a row-major [64][D] tile out of a row-major tensor (K, or V for fp32); the last tile may stick out
-    const unsigned char* base = g + (size_t)kt * G::kKTile;
+    const unsigned char* base = uniform_ptr(g + (size_t)kt * G::kKTile);
     if ((kt + 1) * kBN <= N) {  // one branch per tile, then straight-line loads
 #pragma unroll
       for (int j0 = 0; j0 < kKPer; ++j0) {
@@ -354,7 +354,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   auto issue_k = [&](unsigned char* kb, int kt) { issue_rows(kglob, koff, kb, kt); };
   auto issue_v = [&](unsigned char* vb, int kt) {
     if constexpr (k16) {
-      const unsigned char* base = vglob + (size_t)kt * G::kVTile;  // the transposed copy is padded to whole tiles
+      const unsigned char* base = uniform_ptr(vglob + (size_t)kt * G::kVTile);  // the transposed copy is padded to whole tiles
 #pragma unroll
       for (int j0 = 0; j0 < kVPer; ++j0) {
         const int j = j0 * NW + wave;

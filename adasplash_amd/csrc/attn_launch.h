@@ -1,5 +1,5 @@
-// Host-side dispatch of attn_fwd_kernel over (head dim, alpha mode) for one element type and one of the two
-// instances (kMulti: the one with candidate lists and block bits); each (type, instance) pair is a translation unit of its own.
+// Host-side launch of attn_fwd_kernel for one (element type, head dim, instance) over the alpha modes; kMulti is the
+// instance with candidate lists and block bits.  Each combination is a translation unit of its own (attn_fwd_unit.hip).
 #pragma once
 #include "attn_kernel.h"
 
@@ -25,17 +25,6 @@ template <typename T, int D, bool kMulti> static int launch_attn_am(const AttnPa
   if (am == ATT_15) return launch_attn_one<T, D, ATT_15, kMulti>(p, s);
   if (am == ATT_2) return launch_attn_one<T, D, ATT_2, kMulti>(p, s);
   return launch_attn_one<T, D, ATT_GEN, kMulti>(p, s);
-}
-
-template <typename T, bool kMulti> static int launch_attn(const AttnParams& p, int D, int am, hipStream_t s) {
-  switch (D) {
-    case 16: return launch_attn_am<T, 16, kMulti>(p, am, s);
-    case 32: return launch_attn_am<T, 32, kMulti>(p, am, s);
-    case 64: return launch_attn_am<T, 64, kMulti>(p, am, s);
-    case 128: return launch_attn_am<T, 128, kMulti>(p, am, s);
-    case 256: return launch_attn_am<T, 256, kMulti>(p, am, s);
-  }
-  return 2;
 }
 
 }  // namespace adsp

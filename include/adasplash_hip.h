@@ -49,6 +49,14 @@ typedef enum { ADSP_F32 = 0, ADSP_BF16 = 1, ADSP_F16 = 2 } adsp_dtype;
 /* Library ABI version (bumped when a signature changes). */
 int adsp_version(void);
 
+/*
+ * Identity of the sources this library was built from: the first 16 hex digits of a SHA-256 over the
+ * kernel sources, headers and compiler flags, baked in at build time ("unknown" for a build that did not
+ * pass it).  No counterpart in the reference (pure Python, nothing to go stale); the Python loader compares
+ * it with the tree it sits in so that a library older than its sources cannot be tested or benchmarked.
+ */
+const char* adsp_build_id(void);
+
 /* Static, NUL-terminated description of a status code. */
 const char* adsp_status_string(int status);
 

@@ -145,6 +145,19 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in include/adasplash_hip.h but not exported"
 
 
+def test_library_is_built_from_the_sources_in_the_tree():
+    """The library carries a hash of the kernel sources, headers and flags it was built from; a library older than
+    the sources beside it must not pass for them."""
+    from adasplash_amd import build
+
+    lib = ctypes.CDLL(str(_lib.lib_path()))
+    lib.adsp_build_id.restype = ctypes.c_char_p
+    have = lib.adsp_build_id().decode()
+    assert re.fullmatch(r"[0-9a-f]{16}", have), have
+    assert have == build.source_id(), "libadasplash_hip.so is stale: run `python -m adasplash_amd.build`"
+    assert _lib.build_id() == have  # and the loader, which makes the same comparison, accepts it
+
+
 def test_sizing_helpers_and_status_strings():
     lib = _lib.load()
     assert lib.adsp_version() >= 1
