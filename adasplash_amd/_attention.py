@@ -27,7 +27,7 @@ def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_co
     out = torch.empty_like(q)
     taus = torch.empty((B, Hq, N), device=q.device, dtype=torch.float32)
     bmask = torch.empty((B, Hq, lib.adsp_attn_bmask_words(N)), device=q.device, dtype=torch.int32)
-    ws_bytes = lib.adsp_attn_workspace_bytes(B, Hkv, N, D, dt)
+    ws_bytes = lib.adsp_attn_workspace_bytes(B, Hq, Hkv, N, D, dt)
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
     bits = _varlen_bits(varlen)
     with _lib.device_guard(q.device):

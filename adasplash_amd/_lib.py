@@ -24,7 +24,7 @@ _SIGNATURES = {
     "adsp_status_string": (ctypes.c_char_p, [_i]),
     "adsp_entmax_rows_fwd": (_i, [_vp, _vp, _i64, _i64, _i, _dbl, _i, _i, _i, _vp]),
     "adsp_entmax_rows_bwd": (_i, [_vp, _vp, _vp, _i64, _i64, _i, _dbl, _vp]),
-    "adsp_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "adsp_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "adsp_attn_bmask_words": (_sz, [_i]),
     "adsp_attn_v2_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "adsp_attn_v1_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _dbl, _i, _i, _vp, _sz,

@@ -53,6 +53,8 @@ def units():
             for multi in (0, 1):
                 out.append((f"attn_fwd_{tag}_d{d}_m{multi}", "attn_fwd_unit.hip", base + [f"-DADSP_MULTI={multi}"] + ATTN_FLAGS))
             out.append((f"attn_bwd_{tag}_d{d}", "attn_bwd_unit.hip", base))
+            if tag != "f32" and d in (64, 128):
+                out.append((f"attn_sparse_{tag}_d{d}", "attn_sparse_unit.hip", base + ATTN_FLAGS))
     return out
 
 

@@ -3,6 +3,8 @@
 #include "attn_params.h"
 #include "attn_bwd_params.h"
 #include <math.h>
+#include <stdlib.h>
+#include <string.h>
 #include "../../include/adasplash_hip.h"
 
 namespace adsp {
@@ -16,6 +18,11 @@ namespace adsp {
 ADSP_DECL_TAG(f32)
 ADSP_DECL_TAG(bf16)
 ADSP_DECL_TAG(f16)
+// attn_fwd_sparse_kernel (attn_sparse_unit.hip): 16-bit types, head dims 64 and 128
+int launch_attn_sparse_bf16_d64(const AttnParams&, int, int, hipStream_t);
+int launch_attn_sparse_bf16_d128(const AttnParams&, int, int, hipStream_t);
+int launch_attn_sparse_f16_d64(const AttnParams&, int, int, hipStream_t);
+int launch_attn_sparse_f16_d128(const AttnParams&, int, int, hipStream_t);
 
 typedef int (*attn_fwd_fn)(const AttnParams&, int, hipStream_t);
 typedef int (*attn_bwd_fn)(const AttnBwdParams&, int, hipStream_t);
@@ -36,9 +43,16 @@ static int head_dim_slot(int D) { return D == 16 ? 0 : (D == 32 ? 1 : (D == 64 ?
 // d row as one 16-byte LDS access.
 // A thread moves an 8-key x 8-d block: eight 16-byte loads (one key each), an 8 x 8 transpose of 16-bit values in
 // registers (32 byte permutes), eight 16-byte stores (one d row each).  A 64-key tile takes D threads.
+// `queue` (null, or the eight work counters of the sparse-support forward, which runs behind this kernel on the
+// same stream, followed at word 64 by its two hint counters per K/V head and two over all heads) is cleared on the way.
 __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
                                                         int N, int Npad, int D, const void* varlen, int varlen_bits,
-                                                        int heads) {
+                                                        int heads, uint32_t* queue) {
+  if (queue && blockIdx.x == 0 && threadIdx.x < 8) {
+    if (blockIdx.y == 0) queue[threadIdx.x] = 0u;
+    if (threadIdx.x < 2) queue[64 + 2 * blockIdx.y + threadIdx.x] = 0u;  // the head's pair of hint counters
+    if (blockIdx.y == 0 && threadIdx.x < 2) queue[64 + 2 * gridDim.y + threadIdx.x] = 0u;  // and the pair over all heads
+  }
   const int tiles_per_block = 256 / D;  // D <= 256
   const int t = threadIdx.x % D;
   const int kt = blockIdx.x * tiles_per_block + threadIdx.x / D;
@@ -83,6 +97,39 @@ static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
 static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }
 static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
 
+// Workspace of the forward for the 16-bit types: the key-major copy of V, then -- for the head dims the
+// sparse-support kernel serves -- its work counters, its per-row-block flags and its candidate streams.
+constexpr int kSparseMaxSlots = 1024;                       // workgroups of the persistent kernel
+constexpr size_t kSparseSlotBytes = (size_t)4 * 1472 * 8;   // four waves x 1472 candidates x (score, key)
+struct FwdWorkspace {
+  size_t vt_bytes, queue_off, flags_off, events_off, total;
+  int slots;  // 0: no sparse-support kernel for these dimensions
+};
+static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
+  FwdWorkspace w = {};
+  if (dtype == ADSP_F32) return w;
+  w.vt_bytes = (size_t)B * Hkv * D * npad_of(N) * 2;
+  w.total = w.vt_bytes;
+  if (D == 64 || D == 128) {
+    const long long items = (long long)B * Hq * mblocks_of(N);
+    long long slots = (items + 7) / 8 * 8;
+    if (slots > kSparseMaxSlots) slots = kSparseMaxSlots;
+    w.slots = (int)slots;
+    w.queue_off = align256(w.vt_bytes);
+    w.flags_off = align256(w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8);  // eight counters, then two hint words per K/V head and two more
+    w.events_off = align256(w.flags_off + (size_t)items * 4);
+    w.total = w.events_off + (size_t)slots * kSparseSlotBytes;
+  }
+  return w;
+}
+
+// ADSP_SPARSE=0 in the environment keeps every row block on the dense kernel (for comparisons and tests).
+static bool sparse_enabled() {
+  const char* e = getenv("ADSP_SPARSE");
+  return !(e && strcmp(e, "0") == 0);
+}
+
 static int attn_common(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
                        const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
                        double alpha, int is_causal, int niter, int use_hist, void* workspace, size_t workspace_bytes,
@@ -122,13 +169,33 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.qscale = (float)((alpha - 1.0) / sqrt((double)D));
   const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
 
+  p.block_flags = nullptr;
+  p.queue = nullptr;
+  p.hints = nullptr;
+  p.events = nullptr;
+
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
-    const size_t need = adsp_attn_workspace_bytes(B, Hkv, N, D, dtype);
-    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
+    const FwdWorkspace w = fwd_workspace(B, Hq, Hkv, N, D, dtype);
+    if (!workspace || workspace_bytes < w.total || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
+    unsigned char* ws = (unsigned char*)workspace;
     p.vt = workspace;
+    // Sparse-support kernel first (alpha 1.5 / 2 behind the histogram entry point, no tile statistics asked for): it
+    // serves the row blocks whose supports are short and flags the others for the kernel below.
+    const bool sparse = w.slots > 0 && use_hist && (am == ATT_15 || am == ATT_2) && !tile_counts &&
+                        (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
     hipLaunchKernelGGL(vt_layout_kernel, dim3(vt_layout_blocks(p.Npad, D), (unsigned)(B * Hkv)), dim3(256), 0, s,
-                       (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv);
+                       (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv,
+                       sparse ? (uint32_t*)(ws + w.queue_off) : (uint32_t*)nullptr);
+    if (sparse) {
+      p.queue = (uint32_t*)(ws + w.queue_off);
+      p.hints = p.queue + 64;
+      p.block_flags = (int32_t*)(ws + w.flags_off);
+      p.events = ws + w.events_off;
+      int rc = dtype == ADSP_BF16 ? (D == 64 ? launch_attn_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_sparse_bf16_d128(p, am, w.slots, s))
+                                  : (D == 64 ? launch_attn_sparse_f16_d64(p, am, w.slots, s) : launch_attn_sparse_f16_d128(p, am, w.slots, s));
+      if (rc != 0) return ADSP_ERR_LAUNCH;
+    }
   }
   // The list-carrying instance serves two and more solver steps, and a single step without the histogram (the
   // block-mask variant's, made for sparse supports); the other one no step, or one behind the histogram.
@@ -139,9 +206,9 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
 }
 }  // namespace adsp
 
-extern "C" size_t adsp_attn_workspace_bytes(int B, int Hkv, int N, int D, int dtype) {
-  if (dtype == ADSP_F32 || B <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
-  return (size_t)B * Hkv * D * adsp::npad_of(N) * 2;
+extern "C" size_t adsp_attn_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype) {
+  if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
+  return adsp::fwd_workspace(B, Hq, Hkv, N, D, dtype).total;
 }
 
 extern "C" size_t adsp_attn_bmask_words(int N) {
@@ -223,11 +290,11 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
     const unsigned gx = vt_layout_blocks(p.Npad, D);
     hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hkv)), dim3(256), 0, s, (const uint16_t*)k, kt, N, p.Npad, D,
-                       varlen, varlen_bits, Hkv);
+                       varlen, varlen_bits, Hkv, (uint32_t*)nullptr);
     hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, qt, N, p.Npad, D,
-                       varlen, varlen_bits, Hq);
+                       varlen, varlen_bits, Hq, (uint32_t*)nullptr);
     hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, dot, N, p.Npad,
-                       D, varlen, varlen_bits, Hq);
+                       D, varlen, varlen_bits, Hq, (uint32_t*)nullptr);
     p.kt = kt;
     p.qt = qt;
     p.dot = dot;

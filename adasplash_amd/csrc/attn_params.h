@@ -32,6 +32,12 @@ struct AttnParams {
   float qscale;  // (alpha - 1) / sqrt(D)
   float alpha;
   float c0;  // 1 / (alpha - 1)
+  // Sparse-support path (16-bit types): attn_fwd_sparse_kernel runs first and writes one flag per 128-row block,
+  // 1 = left to attn_fwd_kernel, which skips the others when block_flags is set.
+  int32_t* block_flags;   // [B, Hq, n_mblk], or null: attn_fwd_kernel serves every row block
+  uint32_t* queue;        // eight work counters, one per XCD, zero at launch
+  uint32_t* hints;        // [B * Hkv + 1][2] row blocks {given up, served} per K/V head, then over all heads; zero at launch
+  unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
 };
 
 }  // namespace adsp

@@ -1,0 +1,622 @@
+// Sparse-support forward for 16-bit inputs, alpha = 1.5 / 2 (gfx950): two cheap score walks and no P V product.
+//
+// When a row's support is a few dozen keys out of thousands (unit-variance q and k at head dim 128: about 25 of
+// 8192), every 128 x 64 tile still holds a member of some row's support, so a tile mask skips nothing, yet the
+// output needs only those few keys.  This kernel finds them with two walks over K whose vector work per score is
+// about one instruction, then solves the threshold and forms the output from the short candidate lists:
+//
+//   walk 1  S^T = K Q^T per tile on MFMA; a lane keeps the four largest block maxima of its half of the row's keys.
+//           The threshold of any subset of a row's scores is a lower bound of the row's threshold (f only grows when
+//           entries are added), so a few Newton steps from the left on the row's eight kept values give a rigorous
+//           lower bound `lo` that lies within a few hundredths (in z) of the threshold for such rows.
+//   walk 2  the same products with the accumulators preloaded with -lo; a lane whose eight scores of a 16-key half
+//           block have a positive maximum writes those eight values and the half block's index to its event list in
+//           global memory (a per-workgroup slot of the workspace; the events are a few per cent of the scores).
+//   lists   every lane turns its events into (score - lo, key) pairs in LDS (the K tile buffers, idle by then), the
+//           two lanes of a row run Newton's iteration on them to convergence (from the left: monotone, never past
+//           the root), and the output is the weighted sum of the V rows of the support, read from the row-major V.
+//
+// A row block whose lanes run out of event slots or list room (a dense support) is left to the dense kernel: the
+// kernel writes one flag per row block, and attn_fwd_kernel, launched behind it, serves the flagged ones.
+//
+// The kernel is persistent: a fixed number of workgroups (one event slot each) draw row blocks from per-XCD
+// counters in the same XCD-aware order as the dense kernel, longest causal row blocks first, and help the other
+// XCDs when their own counter runs out.
+#pragma once
+#include "attn_kernel.h"
+
+namespace adsp {
+
+#ifndef ADSP_SPARSE_WAVES
+#define ADSP_SPARSE_WAVES 3
+#endif
+constexpr int kSparseStreamCap = 1472;  // candidates per wave (what SparseGeo::kListCap may be at most)
+
+// acc[2 i] += v[i].lo * p, acc[2 i + 1] += v[i].hi * p for the eight elements of a 16-byte chunk, with the weight given
+// as the pairs plo = (p, 0) and phi = (0, p) of the element type: eight two-term dot products with fp32 accumulation.
+// They are issued as one block that ends in idle cycles: on this part the instruction that follows a v_dot2c must
+// not overwrite one of its source registers (a conversion placed there by the compiler did, and the last of eight
+// sums came out wrong), and the compiler does not keep such writes away by itself.
+template <typename T> __device__ __forceinline__ void dot2_chunk(float (&acc)[8], u32x4 v, uint32_t plo, uint32_t phi);
+#define ADSP_DOT2_CHUNK(OP)                                                                                          \
+  asm volatile(OP " %0, %8, %12\n\t" OP " %1, %8, %13\n\t" OP " %2, %9, %12\n\t" OP " %3, %9, %13\n\t"           \
+               OP " %4, %10, %12\n\t" OP " %5, %10, %13\n\t" OP " %6, %11, %12\n\t" OP " %7, %11, %13\n\ts_nop 3" \
+               : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]),   \
+                 "+v"(acc[7])                                                                                        \
+               : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(plo), "v"(phi))
+template <> __device__ __forceinline__ void dot2_chunk<bf16_t>(float (&acc)[8], u32x4 v, uint32_t plo, uint32_t phi) {
+  ADSP_DOT2_CHUNK("v_dot2c_f32_bf16");
+}
+template <> __device__ __forceinline__ void dot2_chunk<f16_t>(float (&acc)[8], u32x4 v, uint32_t plo, uint32_t phi) {
+  ADSP_DOT2_CHUNK("v_dot2c_f32_f16");
+}
+#undef ADSP_DOT2_CHUNK
+
+// inclusive prefix sum over the wave on the DPP network; all 64 lanes active
+__device__ __forceinline__ int wave_scan_i(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8: a scan inside each row of 16
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+template <typename T, int D> struct SparseGeo {
+  using G = TileGeo<T, D>;
+  static constexpr int kNW = 4;
+  static constexpr int kBM = 32 * kNW;
+  static constexpr int kThreads = 64 * kNW;
+  // two K stages during the walks; afterwards the whole array holds the candidate lists, then the output staging
+  static constexpr int kLds = 2 * G::kKTile > 48 * 1024 ? 2 * G::kKTile : 48 * 1024;
+  static constexpr int kWaveLds = kLds / kNW;
+  static constexpr int kListCap = (kWaveLds - 512) / 8;  // candidates per wave: the lists, then the rows' counters
+  // during walk 2 the LDS behind the two K stages holds a ring of events per wave
+  static constexpr int kRingBytes = (kLds - 2 * G::kKTile) / kNW;
+  static constexpr int kRing = kRingBytes / 36 > 192 ? 192 : kRingBytes / 36;  // events: 8 scores and a tag
+  static_assert(kRing >= 64, "a half block can bring 64 events");
+  static_assert(kListCap <= kSparseStreamCap, "the workspace slot holds kSparseStreamCap candidates per wave");
+};
+
+template <typename T, int D, int AM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE_WAVES, ADSP_SPARSE_WAVES))) void attn_fwd_sparse_kernel(AttnParams p) {
+  using G = TileGeo<T, D>;
+  using SG = SparseGeo<T, D>;
+  using KS = Swz<G::kKRow>;
+  static_assert(G::k16, "16-bit element types only");
+  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  constexpr int NW = SG::kNW, BM = SG::kBM;
+  __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
+  __shared__ int s_item, s_skip;
+  // a lane ran out of event slots, or a wave out of list room.  Two words: the walks write the one of the tile's
+  // parity and read the other one behind the next barrier, so no wave can read a word another one is still setting
+  __shared__ uint32_t s_giveup[2];
+  extern __shared__ uint32_t mask_out[];  // p.mask_words words: key tiles that hold a non-zero probability
+  unsigned char* const k_lds0 = lds_all;
+  unsigned char* const k_lds1 = lds_all + G::kKTile;
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int N = p.N;
+  const int n_mblk = (N + BM - 1) / BM;
+  const int group = p.Hq / p.Hkv;
+  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
+  const long long per_xcd = (total + 7) / 8;
+  const float qs = p.qscale, inv_qs = 1.f / p.qscale;
+  constexpr int kKPer = (G::kKLoads + NW - 1) / NW;
+  constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
+  static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
+
+  int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
+  for (;;) {
+    // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
+    // of this loop they would stay live through both walks, and the walks have no registers to spare.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+    // tile DMA and fragment-read geometry (see attn_fwd_kernel)
+    const uint32_t koff = (uint32_t)((wave * 64 + lane) / KS::kC * G::kKRow + ((((wave * 64 + lane) % KS::kC) ^ KS::sw((wave * 64 + lane) / KS::kC)) << 4));
+    const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
+
+    __syncthreads();  // the previous row block is done with LDS and with s_item
+    if (tid == 0) {
+      int got = -1;
+      while (queues_tried < 8) {
+        const int x = ((int)(blockIdx.x & 7) + queues_tried) & 7;
+        const long long i = (long long)atomicAdd(&p.queue[x], 1u);
+        const long long logical = (long long)x * per_xcd + i;
+        if (i < per_xcd && logical < total) {
+          got = (int)logical;
+          break;
+        }
+        ++queues_tried;
+      }
+      s_item = got;
+      s_skip = 0;
+      if (got >= 0) {  // the K/V head of the row block, as decoded below
+        int unit = got / (group * n_mblk);
+        const int units = p.B * p.Hkv;
+        if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
+        const uint32_t gave_up = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t served = __hip_atomic_load(p.hints + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
+        const uint32_t all_gave_up = __hip_atomic_load(p.hints + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t all_served = __hip_atomic_load(p.hints + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_skip = ((gave_up >= 3u && served == 0u) || (all_gave_up >= 64u && all_served == 0u)) ? 1 : 0;
+      }
+      s_giveup[0] = 0u;
+      s_giveup[1] = 0u;
+    }
+    for (int i = tid; i < p.mask_words; i += SG::kThreads) mask_out[i] = 0u;
+    __syncthreads();
+    const int logical = s_item;
+    if (logical < 0) break;
+
+    // ---- row block -> (batch, kv head, row block, head in group), as in attn_fwd_kernel ---------------------
+    const int hg = logical % group;
+    const int mi = (logical / group) % n_mblk;
+    int bkv = logical / (group * n_mblk);
+    {
+      const int units = p.B * p.Hkv;
+      if (units % 8 == 0) bkv = (bkv % (units / 8)) * 8 + bkv / (units / 8);
+    }
+    const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
+    const int h = kvh * group + hg;
+    const int mblk = n_mblk - 1 - mi;
+    const int m0 = mblk * BM;
+    int L = N;
+    if (p.varlen) {
+      long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
+      L = (int)(l < 0 ? 0 : (l > N ? N : l));
+    }
+    int32_t* const flag = p.block_flags + ((size_t)(b * p.Hq + h) * n_mblk + mblk);
+    // Row blocks of one K/V head tend to share their fate: once a few of them were given up and none succeeded, the
+    // rest go to the dense kernel unseen (a hint only: thread 0 read the counters, without any ordering, above).
+    uint32_t* const hint = p.hints + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
+    const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
+    const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
+    int32_t* const bmask_out = p.bmask ? p.bmask + ((size_t)(b * p.Hq + h) * p.n_mblk + (size_t)mblk) * p.mask_words : nullptr;
+    const int qi = m0 + wave * 32 + lq;
+
+    if (m0 >= L) {  // row block entirely inside the padding: zero rows, empty mask
+      if (bmask_out)
+        for (int i = tid; i < p.mask_words; i += SG::kThreads) bmask_out[i] = 0;
+      constexpr int kRowDw = D * 2 / 4;
+      uint32_t* o32 = reinterpret_cast<uint32_t*>(p.out) + (qo_base + (size_t)m0 * D) * 2 / 4;
+      const int rows = (N - m0) < BM ? (N - m0) : BM;
+      for (int i = tid; i < rows * kRowDw; i += SG::kThreads) o32[i] = 0u;
+      if (tid == 0) *flag = 0;
+      continue;
+    }
+
+    if (s_skip) {
+      if (tid == 0) *flag = 1;
+      continue;
+    }
+    const int row_hi = (m0 + BM < L ? m0 + BM : L);
+    const int nt = p.causal ? (row_hi + kBN - 1) / kBN : (L + kBN - 1) / kBN;
+    const int lim = p.causal ? (qi < L - 1 ? qi : L - 1) : L - 1;
+    const int wave_row0 = m0 + wave * 32;
+    const bool live = qi < L;
+
+    // ---- Q fragments; rows past the valid length are zero (their scores are never used) ----------------------
+    uint32_t qf[G::kQRegs];
+    {
+      const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = live ? raw[e] : 0u;
+      }
+    }
+
+    const unsigned char* kglob = reinterpret_cast<const unsigned char*>(p.k) + kv_base * 2;
+    auto issue_k = [&](unsigned char* lds, int kt) {
+      const unsigned char* base = uniform_ptr(kglob + (size_t)kt * G::kKTile);
+      if ((kt + 1) * kBN <= N) {
+#pragma unroll
+        for (int j0 = 0; j0 < kKPer; ++j0) dma16s(base + j0 * (NW * 1024), koff, lds + (j0 * NW + wave) * 1024);
+      } else {  // the last tile sticks out of the tensor: rows past the end are masked later, any valid row will do
+        const unsigned char* g = uniform_ptr(kglob);
+        const int row0 = (int)(koff / G::kKRow);
+        const uint32_t coff = koff % G::kKRow;
+#pragma unroll
+        for (int j0 = 0; j0 < kKPer; ++j0) {
+          int gk = kt * kBN + row0 + j0 * (NW * 64 / KS::kC);
+          gk = gk < N ? gk : N - 1;
+          dma16s(g, (uint32_t)gk * (uint32_t)G::kKRow + coff, lds + (j0 * NW + wave) * 1024);
+        }
+      }
+    };
+    // body(kt, tile) over all key tiles of the row block, K double-buffered; stops when a lane gave up
+    auto walk = [&](auto&& body) {
+      __syncthreads();
+      int cur = 0;
+      issue_k(k_lds0, 0);
+      for (;;) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        __syncthreads();
+        if (s_giveup[(cur + 1) & 1]) break;  // set while the previous tile was worked on
+        if (cur + 1 < nt) issue_k(k_lds1, cur + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, k_lds0);
+        if (++cur >= nt) break;
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (s_giveup[(cur + 1) & 1]) break;
+        if (cur + 1 < nt) issue_k(k_lds0, cur + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, k_lds1);
+        if (++cur >= nt) break;
+      }
+    };
+    // S^T of one tile (two 32-key blocks), accumulators preloaded with `init`; f(s0, s1) unless no row of the wave
+    // sees the tile.  Scores past a row's last valid key are -inf.
+    auto for_tile = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
+      if (p.causal && kt * kBN > wave_row0 + 31) return;
+      const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
+      f32x16 s0, s1;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s0[i] = init;
+        s1[i] = init;
+      }
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
+      asm volatile("" : "+v"(ka));
+      u32x4 a0[D / 16], a1[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a0[ks] = lds_read16(ka ^ (ks << 5));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a1[ks] = lds_read16(ka ^ (ks << 5), 32 * G::kKRow);
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s0 = mfma_16bit<T>(a0[ks], bq, s0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s1 = mfma_16bit<T>(a1[ks], bq, s1);
+      }
+      if (need_mask) {
+        const int jb = kt * kBN + 4 * lh;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s0[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? s0[i] : -INFINITY;
+          s1[i] = (jb + 32 + 8 * (i >> 2) + (i & 3) <= lim) ? s1[i] : -INFINITY;
+        }
+      }
+      f(s0, s1);
+    };
+
+    // ---- walk 1: the four largest block maxima of the lane's keys ---------------------------------------------
+    float t1 = -INFINITY, t2 = -INFINITY, t3 = -INFINITY, t4 = -INFINITY;
+    auto keep_top = [&](float x) {
+      const float n2 = __builtin_amdgcn_fmed3f(t1, t2, x), n3 = __builtin_amdgcn_fmed3f(t2, t3, x), n4 = __builtin_amdgcn_fmed3f(t3, t4, x);
+      t1 = fmaxf(t1, x);
+      t2 = n2;
+      t3 = n3;
+      t4 = n4;
+    };
+    // A flat score distribution (a support of hundreds of keys) shows early: most block maxima lie close to the
+    // running maximum.  Tiles 6 .. 11 are counted; if more than half of their (lane, block) maxima lie within 1/4 (in
+    // z) of the lane's running maximum, the row block is given up before the walk is over.  A heuristic that only
+    // decides which kernel does the work.
+    int near_cnt = 0;
+    walk([&](int kt, const unsigned char* kt_lds) {
+      for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
+        float m0v = s0[0], m1v = s1[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) {
+          m0v = fmaxf(m0v, s0[i]);
+          m1v = fmaxf(m1v, s1[i]);
+        }
+        keep_top(m0v);
+        keep_top(m1v);
+        if (kt >= 6 && kt < 12) {
+          const float near = t1 - 0.25f * inv_qs;
+          near_cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && m0v > near)) + __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && m1v > near));
+          if (kt == 11 && near_cnt > 6 * 128 / 2 && lane == 0) s_giveup[1] = 1u;
+        }
+      });
+    });
+
+    __syncthreads();
+    if (s_giveup[0] | s_giveup[1]) {  // a flat score distribution: the dense kernel's case
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(hint, 1u);
+        atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
+      }
+      continue;
+    }
+    // ---- lower bound of the row's threshold from its eight kept values (raw score units) --------------------
+    // f(t) = qs^2 sum (r - t)_+^2 - 1 (alpha 1.5) or qs sum (r - t)_+ - 1 (alpha 2) is convex and decreasing and
+    // f(max - 1 / qs) >= 0, so Newton from there approaches the subset's root from the left and never passes it.
+    float lo_raw;
+    {
+      float r[8] = {t1, t2, t3, t4, __shfl_xor(t1, 32, 64), __shfl_xor(t2, 32, 64), __shfl_xor(t3, 32, 64), __shfl_xor(t4, 32, 64)};
+      const float rmax = fmaxf(r[0], r[4]);
+      float t = rmax - inv_qs;
+      const float target = (AM == ATT_15) ? inv_qs * inv_qs : inv_qs;
+#pragma unroll 1
+      for (int it = 0; it < 8; ++it) {
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float u = fmaxf(r[i] - t, 0.f);
+          if constexpr (AM == ATT_15) {
+            a0 = fmaf(u, u, a0);
+            a1 += u;
+          } else {
+            a0 += u;
+            a1 += u > 0.f ? 1.f : 0.f;
+          }
+        }
+        const float step = (AM == ATT_15) ? (a0 - target) / (2.f * a1) : (a0 - target) / a1;
+        t += (a1 > 0.f && step > 0.f) ? step : 0.f;
+      }
+      // the margin covers the rounding of the iteration; rows past the valid length take no part in walk 2
+      lo_raw = t - (1e-5f * inv_qs + 1e-6f * fabsf(rmax));
+      lo_raw = (live && rmax > -INFINITY) ? lo_raw : INFINITY;
+    }
+
+    // ---- walk 2: collect the scores above the bound -------------------------------------------------------------
+    // A lane whose eight scores of a 16-key half block have a positive maximum puts them, with a tag, into the wave's
+    // ring in LDS (slots are handed out with a ballot: no atomics).  When the ring is full the wave empties it, one
+    // event per lane: the positive entries go to the wave's candidate stream in global memory as (score - lo, key and
+    // row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
+    float* const ring = reinterpret_cast<float*>(lds_all + 2 * G::kKTile + wave * SG::kRingBytes);
+    uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
+    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)SG::kListCap;
+    int ring_n = 0, stream_n = 0;  // wave-uniform
+    // (kt: the tile being worked on; a stream that fills faster than the tiles go by will not last: give up early)
+    auto flush = [&](int parity, int kt) {
+      for (int e0 = 0; e0 < ring_n; e0 += 64) {
+        const int e = e0 + lane;
+        const bool has = e < ring_n;
+        f32x4 w0 = {0.f, 0.f, 0.f, 0.f}, w1 = {0.f, 0.f, 0.f, 0.f};
+        uint32_t tag = 0u;
+        if (has) {
+          w0 = *reinterpret_cast<const f32x4*>(ring + e * 8);
+          w1 = *reinterpret_cast<const f32x4*>(ring + e * 8 + 4);
+          tag = ring_tag[e];
+        }
+        int c = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c += (w0[i] > 0.f ? 1 : 0) + (w1[i] > 0.f ? 1 : 0);
+        const int incl = wave_scan_i(c);
+        const int total_c = __builtin_amdgcn_readlane(incl, 63);
+        if (stream_n + total_c > SG::kListCap || (long long)(stream_n + total_c) * nt > (long long)SG::kListCap * (kt + 16)) {
+          if (lane == 0) s_giveup[parity] = 1u;
+        } else {
+          // producer lane = tag & 63: row (tag & 31), key half (tag >> 5) & 1; half block (tag >> 6) & 3 of tile tag >> 8
+          const uint32_t key0 = (tag >> 8) * kBN + ((tag >> 6) & 3u) * 16 + 4 * ((tag >> 5) & 1u);
+          const uint32_t rowbits = (tag & 31u) << 20;
+          uint2* dst = stream + stream_n + (incl - c);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float x = i < 4 ? w0[i & 3] : w1[i & 3];
+            if (x > 0.f) {
+              *dst = uint2{__builtin_bit_cast(uint32_t, x), (key0 + 8 * (i >> 2) + (i & 3)) | rowbits};
+              ++dst;
+            }
+          }
+          stream_n += total_c;
+        }
+      }
+      ring_n = 0;
+    };
+    auto collect = [&](const f32x16& s, int first, float hmax, uint32_t tag, int kt) {
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(hmax > 0.f);
+      if (m != 0ull) {
+        const int c = __builtin_popcountll(m);
+        if (ring_n + c > SG::kRing) flush(kt & 1, kt);
+        if (hmax > 0.f) {
+          const int slot = ring_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+          f32x4 w0 = {s[first], s[first + 1], s[first + 2], s[first + 3]};
+          f32x4 w1 = {s[first + 4], s[first + 5], s[first + 6], s[first + 7]};
+          *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
+          *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
+          ring_tag[slot] = (tag << 6) | (uint32_t)lane;
+        }
+        ring_n += c;
+      }
+    };
+    walk([&](int kt, const unsigned char* kt_lds) {
+      for_tile(kt, kt_lds, -lo_raw, [&](const f32x16& s0, const f32x16& s1) {
+        float h00 = s0[0], h01 = s0[8], h10 = s1[0], h11 = s1[8];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+          h00 = fmaxf(h00, s0[i]);
+          h01 = fmaxf(h01, s0[8 + i]);
+          h10 = fmaxf(h10, s1[i]);
+          h11 = fmaxf(h11, s1[8 + i]);
+        }
+        collect(s0, 0, h00, (uint32_t)(kt * 4 + 0), kt);
+        collect(s0, 8, h01, (uint32_t)(kt * 4 + 1), kt);
+        collect(s1, 0, h10, (uint32_t)(kt * 4 + 2), kt);
+        collect(s1, 8, h11, (uint32_t)(kt * 4 + 3), kt);
+      });
+    });
+    flush(0, nt);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
+    __syncthreads();                      // every wave has left the K tiles: LDS becomes the lists
+    if (s_giveup[0] | s_giveup[1]) {
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(hint, 1u);
+        atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
+      }
+      continue;
+    }
+
+    // ---- the wave's stream -> per-row lists in its share of LDS (a counting sort by row) ----------------------------
+    unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
+    uint2* const lst = reinterpret_cast<uint2*>(wave_lds);                                   // kListCap entries
+    uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 8);     // 32 counters
+    uint32_t* const row_start = row_cnt + 32;                                                // 33 offsets
+    float* const row_inv = reinterpret_cast<float*>(row_start + 33);                         // 32 x 1 / sum p
+    if (lane < 32) row_cnt[lane] = 0u;
+    {
+      constexpr int kPer = (SG::kListCap + 63) / 64;
+      uint2 ent[kPer];
+      uint32_t pos[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        ent[j] = uint2{0u, 0u};
+        if (e < stream_n) ent[j] = stream[e];
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        pos[j] = 0u;
+        if (e < stream_n) pos[j] = atomicAdd(&row_cnt[(ent[j].y >> 20) & 31u], 1u);
+      }
+      {
+        const int c = lane < 32 ? (int)row_cnt[lane] : 0;
+        const int incl = wave_scan_i(c);
+        if (lane < 32) row_start[lane] = (uint32_t)(incl - c);
+        if (lane == 31) row_start[32] = (uint32_t)incl;
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        if (e < stream_n) lst[row_start[(ent[j].y >> 20) & 31u] + pos[j]] = uint2{ent[j].x, ent[j].y & 0xfffffu};
+      }
+    }
+
+    // ---- threshold: Newton from the left on the row's candidates (its two lanes take alternate entries) -----------
+    const int row_lo = (int)row_start[lq], row_end = (int)row_start[lq + 1];
+    float t = 0.f;  // threshold minus lo, raw units
+    {
+      const float target = (AM == ATT_15) ? inv_qs * inv_qs : inv_qs;
+      for (int it = 0; it < 24; ++it) {
+        float a0 = 0.f, a1 = 0.f;
+        for (int e = row_lo + lh; e < row_end; e += 2) {
+          const float u = fmaxf(__builtin_bit_cast(float, lst[e].x) - t, 0.f);
+          if constexpr (AM == ATT_15) {
+            a0 = fmaf(u, u, a0);
+            a1 += u;
+          } else {
+            a0 += u;
+            a1 += u > 0.f ? 1.f : 0.f;
+          }
+        }
+        a0 += __shfl_xor(a0, 32, 64);
+        a1 += __shfl_xor(a1, 32, 64);
+        const float step = (AM == ATT_15) ? (a0 - target) / (2.f * a1) : (a0 - target) / a1;
+        const bool move = a1 > 0.f && step > 1e-7f * inv_qs;
+        t += move ? step : 0.f;
+        if (__builtin_amdgcn_ballot_w64(move) == 0ull) break;
+      }
+    }
+    // scores -> probabilities (not yet normalised): the row's first lane rewrites its list in place, keeping only the
+    // support; 1 / sum per row
+    {
+      float psum = 0.f;
+      int w = row_lo;
+      if (lh == 0) {
+        for (int e = row_lo; e < row_end; ++e) {
+          const uint2 en = lst[e];
+          const float u = __builtin_bit_cast(float, en.x) - t;
+          if (u > 0.f) {
+            const float pv = (AM == ATT_15) ? u * u : u;
+            lst[w] = uint2{__builtin_bit_cast(uint32_t, pv), en.y};
+            ++w;
+            psum += pv;
+          }
+        }
+        row_cnt[lq] = (uint32_t)(w - row_lo);
+        row_inv[lq] = (live && psum > 0.f) ? 1.f / psum : 0.f;
+        if (live && p.taus) p.taus[(size_t)(b * p.Hq + h) * N + qi] = (lo_raw + t) * qs;
+      }
+    }
+
+    // ---- output: a group of D / 8 lanes per row, each lane 8 columns; the V rows of a row's support are fetched
+    // kDepth at a time (all in flight together), weighted, summed, and the row is stored with 16-byte accesses.  The
+    // weights enter the two-term dot product as (p, 0) and (0, p) pairs of the element type, i.e. rounded to it, as
+    // the P operand of the dense kernel's MFMA is. ---------------------------------------------------------------------
+    {
+      constexpr int kLPR = D / 8;         // lanes per row
+      constexpr int kGroups = 64 / kLPR;  // rows in progress per wave
+      constexpr int kDepth = 8;
+      const int grp = lane / kLPR, col = lane % kLPR;
+      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
+      unsigned char* obase = reinterpret_cast<unsigned char*>(p.out) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
+      for (int r0 = 0; r0 < 32; r0 += kGroups) {
+        const int r = r0 + grp;
+        const int e_lo = (int)row_start[r], e_hi = e_lo + (int)row_cnt[r];
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+        for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+          u32x4 vv[kDepth];
+          uint32_t pw[kDepth];
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            pw[j] = 0u;
+            vv[j] = u32x4{0u, 0u, 0u, 0u};
+            if (eb + j < e_hi) {
+              const uint2 en = lst[eb + j];
+              pw[j] = en.x;
+              vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)en.y * (D * 2));
+              if (col == 0) atomicOr(&mask_out[(en.y / kBN) >> 5], 1u << ((en.y / kBN) & 31));
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            const uint32_t plo = pack2<T>(__builtin_bit_cast(float, pw[j]), 0.f), phi = plo << 16;
+            dot2_chunk<T>(acc, vv[j], plo, phi);
+          }
+        }
+        const float inv = row_inv[r];
+        if (wave_row0 + r < N) {
+          u32x4 w = {pack2<T>(acc[0] * inv, acc[1] * inv), pack2<T>(acc[2] * inv, acc[3] * inv),
+                     pack2<T>(acc[4] * inv, acc[5] * inv), pack2<T>(acc[6] * inv, acc[7] * inv)};
+          *reinterpret_cast<u32x4*>(obase + (size_t)r * (D * 2)) = w;
+        }
+      }
+    }
+    __syncthreads();  // every wave's tile marks are in
+    if (bmask_out)
+      for (int i = tid; i < p.mask_words; i += SG::kThreads) bmask_out[i] = (int32_t)mask_out[i];
+    if (tid == 0) {
+      *flag = 0;
+      atomicAdd(hint + 1, 1u);
+      atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);
+    }
+  }
+}
+
+// Workgroups to launch: as many as fit the device at once (each owns one event slot), at most `max_slots`.
+template <typename T, int D, int AM> static int launch_attn_sparse_one(const AttnParams& p, int max_slots, hipStream_t s) {
+  using SG = SparseGeo<T, D>;
+  auto kern = attn_fwd_sparse_kernel<T, D, AM>;
+  static int per_cu = 0, n_cu = 0;  // (one device family per process: gfx950)
+  const size_t dyn = (size_t)p.mask_words * sizeof(uint32_t);
+  if (per_cu == 0) {
+    int dev = 0, blocks = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 2;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kern, SG::kThreads, dyn) != hipSuccess || blocks <= 0) blocks = 1;
+    n_cu = prop.multiProcessorCount;
+    per_cu = blocks;
+  }
+  long long grid = (long long)per_cu * n_cu;
+  if (grid > max_slots) grid = max_slots;
+  grid = grid / 8 * 8;  // the same number of workgroups on every XCD
+  if (grid < 8) grid = 8;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(SG::kThreads), dyn, s, p);
+  return 0;
+}
+
+template <typename T, int D> static int launch_attn_sparse(const AttnParams& p, int am, int max_slots, hipStream_t s) {
+  if (am == ATT_15) return launch_attn_sparse_one<T, D, ATT_15>(p, max_slots, s);
+  if (am == ATT_2) return launch_attn_sparse_one<T, D, ATT_2>(p, max_slots, s);
+  return 2;
+}
+
+}  // namespace adsp

@@ -79,10 +79,12 @@ int adsp_entmax_rows_bwd(const void* y, const void* dy, void* dx, int64_t rows, 
                          double alpha, void* stream);
 
 /*
- * Bytes of scratch the attention entry points need for these dimensions (a key-major copy of V for
- * the 16-bit types; 0 for fp32).  The buffer must be 256-byte aligned device memory.
+ * Bytes of scratch the forward entry points need for these dimensions; 0 for fp32.  For the 16-bit types: a
+ * key-major copy of V and, at head dims 64 and 128, the work counters, row-block flags and event slots of the
+ * sparse-support kernel (up to 1024 slots of 46 KiB).  The buffer must be 16-byte aligned device memory; its
+ * contents need not survive between calls.  For the block-mask variant pass Hq = Hkv = H.
  */
-size_t adsp_attn_workspace_bytes(int B, int Hkv, int N, int D, int dtype);
+size_t adsp_attn_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
 
 /* Number of int32 words per (batch, head) the block mask needs: n_row_blocks * words_per_row. */
 size_t adsp_attn_bmask_words(int N);
