@@ -43,16 +43,12 @@ static int head_dim_slot(int D) { return D == 16 ? 0 : (D == 32 ? 1 : (D == 64 ?
 // d row as one 16-byte LDS access.
 // A thread moves an 8-key x 8-d block: eight 16-byte loads (one key each), an 8 x 8 transpose of 16-bit values in
 // registers (32 byte permutes), eight 16-byte stores (one d row each).  A 64-key tile takes D threads.
-// `queue` (null, or the eight work counters of the sparse-support forward, which runs behind this kernel on the
-// same stream, followed at word 64 by its two hint counters per K/V head and two over all heads) is cleared on the way.
+// `ctrl` (null, or the control words of the sparse-support forward, which ran before this kernel on the same stream):
+// the copy is only needed by the dense kernel, so it is skipped when that kernel has no row block to serve.
 __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
                                                         int N, int Npad, int D, const void* varlen, int varlen_bits,
-                                                        int heads, uint32_t* queue) {
-  if (queue && blockIdx.x == 0 && threadIdx.x < 8) {
-    if (blockIdx.y == 0) queue[threadIdx.x] = 0u;
-    if (threadIdx.x < 2) queue[64 + 2 * blockIdx.y + threadIdx.x] = 0u;  // the head's pair of hint counters
-    if (blockIdx.y == 0 && threadIdx.x < 2) queue[64 + 2 * gridDim.y + threadIdx.x] = 0u;  // and the pair over all heads
-  }
+                                                        int heads, const uint32_t* ctrl) {
+  if (ctrl && ctrl[kCtrlFlagged] == 0u && ctrl[kCtrlAllDense] == 0u) return;
   const int tiles_per_block = 256 / D;  // D <= 256
   const int t = threadIdx.x % D;
   const int kt = blockIdx.x * tiles_per_block + threadIdx.x / D;
@@ -96,6 +92,90 @@ static unsigned vt_layout_blocks(int Npad, int D) {  // 256 / D tiles of 64 keys
 static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
 static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }
 static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
+
+// Control words of the sparse-support forward (the `queue` pointer of AttnParams): eight work counters, the number
+// of row blocks it left to the dense kernel, a word saying that the probe below predicts every K/V head to be dense; from word
+// 64 on two hint counters {given up, served} per K/V head and one more pair over all heads.
+//
+// attn_probe_kernel clears them and looks at a sample of each K/V head's scores (one workgroup per head: four long
+// query rows of the group's first head against 256 evenly spaced keys): from the sample's variance and the row
+// length, the support a Gaussian score distribution would have follows in closed form (n s^2 g(a) = 1 with
+// g(a) = (1 + a^2) Q(a) - a phi(a) for alpha = 1.5, n s h(a) = 1 with h(a) = phi(a) - a Q(a) for alpha = 2; support
+// n Q(a)).  Heads whose predicted support is far beyond what the candidate lists hold are marked as given up, so the
+// sparse-support kernel does not spend a walk on finding that out.  The prediction only decides which kernel does
+// the work; a head it gets wrong is caught by the kernel's own checks.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, int am) {
+  __shared__ float qrows[4][256];
+  __shared__ float red[4][2][4];
+  const int u = blockIdx.x, tid = threadIdx.x;
+  const int units = p.B * p.Hkv;
+  uint32_t* const ctrl = p.queue;
+  if (u == 0 && tid < 10) ctrl[tid] = 0u;
+  if (u == 0 && tid < 2) ctrl[64 + 2 * units + tid] = 0u;
+  if (tid < 2) ctrl[64 + 2 * u + tid] = 0u;
+  const int b = u / p.Hkv, kvh = u % p.Hkv, group = p.Hq / p.Hkv;
+  int L = p.N;
+  if (p.varlen) {
+    long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
+    L = (int)(l < 0 ? 0 : (l > p.N ? p.N : l));
+  }
+  if (L < 2048) return;  // short sequences: finding out in the kernel costs little
+  int rows[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rows[j] = L - 1 - j * (L / 16);
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)(b * p.Hq + kvh * group) * p.N) * D;
+  for (int i = tid; i < 4 * D; i += 256) {
+    const uint32_t w = qbase[(size_t)rows[i / D] * D + i % D];
+    qrows[i / D][i % D] = elem_traits<T>::kIsBf16 ? bf16_bits_to_float(w) : f16_bits_to_float(w);
+  }
+  __syncthreads();
+  const int span = (p.causal ? rows[3] + 1 : L);
+  const int key = (int)(((long long)tid * span) / 256);
+  const uint16_t* krow = reinterpret_cast<const uint16_t*>(p.k) + ((size_t)(b * p.Hkv + kvh) * p.N + key) * D;
+  float dot[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int d = 0; d < D; d += 8) {
+    const u32x4 w = *reinterpret_cast<const u32x4*>(krow + d);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float lo = unpack_lo<T>(w[e]), hi = unpack_hi<T>(w[e]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dot[j] = fmaf(lo, qrows[j][d + 2 * e], fmaf(hi, qrows[j][d + 2 * e + 1], dot[j]));
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float z = dot[j] * p.qscale;
+    const float s1 = wave_sum(z), s2 = wave_sum(z * z);
+    if ((tid & 63) == 0) {
+      red[tid >> 6][0][j] = s1;
+      red[tid >> 6][1][j] = s2;
+    }
+  }
+  __syncthreads();
+  if (tid >= 4) return;
+  {  // threads 0 .. 3: one sampled row each
+    const int j = tid;
+    const float s1 = red[0][0][j] + red[1][0][j] + red[2][0][j] + red[3][0][j];
+    const float s2 = red[0][1][j] + red[1][1][j] + red[2][1][j] + red[3][1][j];
+    const float mean = s1 / 256.f, var = fmaxf(s2 / 256.f - mean * mean, 0.f), sd = sqrtf(var);
+    const float n = (float)(p.causal ? rows[j] + 1 : L);
+    float lo = -2.f, hi = 7.f;
+    for (int it = 0; it < 14; ++it) {
+      const float a = 0.5f * (lo + hi);
+      const float Q = 0.5f * erfcf(a * 0.70710678f), phi = 0.39894228f * __expf(-0.5f * a * a);
+      const float f = am == ATT_2 ? n * sd * (phi - a * Q) : n * var * ((1.f + a * a) * Q - a * phi);
+      if (f > 1.f) lo = a;
+      else hi = a;
+    }
+    const float support = n * 0.5f * erfcf(0.5f * (lo + hi) * 0.70710678f);
+    red[0][0][j] = support > 40.f ? 1.f : 0.f;
+  }
+  // (the four threads are lanes of one wave: their LDS writes are in order before the read below)
+  const int dense_rows = (int)(red[0][0][0] + red[0][0][1] + red[0][0][2] + red[0][0][3]);
+  if (tid != 0) return;
+  if (dense_rows >= 3) ctrl[64 + 2 * u] = 1u << 20;  // (the sparse kernel counts the marked heads itself)
+}
 
 // Workspace of the forward for the 16-bit types: the key-major copy of V, then -- for the head dims the
 // sparse-support kernel serves -- its work counters, its per-row-block flags and its candidate streams.
@@ -184,18 +264,21 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
     // serves the row blocks whose supports are short and flags the others for the kernel below.
     const bool sparse = w.slots > 0 && use_hist && (am == ATT_15 || am == ATT_2) && !tile_counts &&
                         (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
-    hipLaunchKernelGGL(vt_layout_kernel, dim3(vt_layout_blocks(p.Npad, D), (unsigned)(B * Hkv)), dim3(256), 0, s,
-                       (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv,
-                       sparse ? (uint32_t*)(ws + w.queue_off) : (uint32_t*)nullptr);
     if (sparse) {
       p.queue = (uint32_t*)(ws + w.queue_off);
       p.hints = p.queue + 64;
       p.block_flags = (int32_t*)(ws + w.flags_off);
       p.events = ws + w.events_off;
+      if (dtype == ADSP_BF16) hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
+      else hipLaunchKernelGGL(attn_probe_kernel<f16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
       int rc = dtype == ADSP_BF16 ? (D == 64 ? launch_attn_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_sparse_bf16_d128(p, am, w.slots, s))
                                   : (D == 64 ? launch_attn_sparse_f16_d64(p, am, w.slots, s) : launch_attn_sparse_f16_d128(p, am, w.slots, s));
       if (rc != 0) return ADSP_ERR_LAUNCH;
     }
+    // the key-major copy of V serves the dense kernel only
+    hipLaunchKernelGGL(vt_layout_kernel, dim3(vt_layout_blocks(p.Npad, D), (unsigned)(B * Hkv)), dim3(256), 0, s,
+                       (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv,
+                       (const uint32_t*)p.queue);
   }
   // The list-carrying instance serves two and more solver steps, and a single step without the histogram (the
   // block-mask variant's, made for sparse supports); the other one no step, or one behind the histogram.
@@ -290,11 +373,11 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
     const unsigned gx = vt_layout_blocks(p.Npad, D);
     hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hkv)), dim3(256), 0, s, (const uint16_t*)k, kt, N, p.Npad, D,
-                       varlen, varlen_bits, Hkv, (uint32_t*)nullptr);
+                       varlen, varlen_bits, Hkv, (const uint32_t*)nullptr);
     hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, qt, N, p.Npad, D,
-                       varlen, varlen_bits, Hq, (uint32_t*)nullptr);
+                       varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
     hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, dot, N, p.Npad,
-                       D, varlen, varlen_bits, Hq, (uint32_t*)nullptr);
+                       D, varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
     p.kt = kt;
     p.qt = qt;
     p.dot = dot;

@@ -230,7 +230,9 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   const int mblk = n_mblk - 1 - mi;
   const int m0 = mblk * BM;
   // behind the sparse-support kernel: only the row blocks it left over (its flags are per 128 rows, BM here)
-  if (p.block_flags && p.block_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] == 0) return;
+  if (p.block_flags && p.queue[kCtrlAllDense] == 0u &&
+      (p.queue[kCtrlFlagged] == 0u || p.block_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] == 0))
+    return;
 
   const int N = p.N;
   int L = N;

@@ -10,6 +10,9 @@ constexpr int kAttnBins = 8;     // histogram bins of the attention solver
 constexpr int kMaskWords = 512;  // tile-mask capacity per row block: 512 * 32 tiles * 64 keys = 1M keys
 
 enum AttnAlphaMode { ATT_15 = 0, ATT_2 = 1, ATT_GEN = 2 };
+// control words of the sparse-support forward behind the eight work counters (AttnParams::queue)
+constexpr int kCtrlFlagged = 8;     // row blocks left to the dense kernel
+constexpr int kCtrlAllDense = 9;    // set by the sparse kernel when every K/V head was predicted dense: it served nothing
 
 struct AttnParams {
   const void* q;
@@ -35,7 +38,7 @@ struct AttnParams {
   // Sparse-support path (16-bit types): attn_fwd_sparse_kernel runs first and writes one flag per 128-row block,
   // 1 = left to attn_fwd_kernel, which skips the others when block_flags is set.
   int32_t* block_flags;   // [B, Hq, n_mblk], or null: attn_fwd_kernel serves every row block
-  uint32_t* queue;        // eight work counters, one per XCD, zero at launch
+  uint32_t* queue;        // eight work counters, one per XCD, then the two control words above; zero at launch
   uint32_t* hints;        // [B * Hkv + 1][2] row blocks {given up, served} per K/V head, then over all heads; zero at launch
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
 };

@@ -107,7 +107,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
   static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
 
+  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all row blocks
+    const int units = p.B * p.Hkv;
+    int unmarked = 0;
+    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints[2 * u] < (1u << 20) ? 1 : 0;
+    if (__syncthreads_count(unmarked) == 0) {
+      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue[kCtrlAllDense] = 1u;
+      return;
+    }
+  }
   int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
+  int known_unit = -1;   // thread 0: the K/V head whose hint counters it has last seen (or set) as served
   for (;;) {
     // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
     // of this loop they would stay live through both walks, and the walks have no registers to spare.
@@ -137,12 +147,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         int unit = got / (group * n_mblk);
         const int units = p.B * p.Hkv;
         if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
-        const uint32_t gave_up = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t served = __hip_atomic_load(p.hints + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
-        const uint32_t all_gave_up = __hip_atomic_load(p.hints + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t all_served = __hip_atomic_load(p.hints + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_skip = ((gave_up >= 3u && served == 0u) || (all_gave_up >= 64u && all_served == 0u)) ? 1 : 0;
+        if (unit != known_unit) {
+          const uint32_t gave_up = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t served = __hip_atomic_load(p.hints + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
+          const uint32_t all_gave_up = __hip_atomic_load(p.hints + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t all_served = __hip_atomic_load(p.hints + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          s_skip = ((gave_up >= 3u && served == 0u) || (all_gave_up >= 64u && all_served == 0u)) ? 1 : 0;
+          if (served > 0u) known_unit = unit;
+        }
       }
       s_giveup[0] = 0u;
       s_giveup[1] = 0u;
@@ -190,7 +203,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     }
 
     if (s_skip) {
-      if (tid == 0) *flag = 1;
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(&p.queue[kCtrlFlagged], 1u);
+      }
       continue;
     }
     const int row_hi = (m0 + BM < L ? m0 + BM : L);
@@ -326,6 +342,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     if (s_giveup[0] | s_giveup[1]) {  // a flat score distribution: the dense kernel's case
       if (tid == 0) {
         *flag = 1;
+        atomicAdd(&p.queue[kCtrlFlagged], 1u);
         atomicAdd(hint, 1u);
         atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
       }
@@ -446,6 +463,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     if (s_giveup[0] | s_giveup[1]) {
       if (tid == 0) {
         *flag = 1;
+        atomicAdd(&p.queue[kCtrlFlagged], 1u);
         atomicAdd(hint, 1u);
         atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
       }
@@ -585,8 +603,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       for (int i = tid; i < p.mask_words; i += SG::kThreads) bmask_out[i] = (int32_t)mask_out[i];
     if (tid == 0) {
       *flag = 0;
-      atomicAdd(hint + 1, 1u);
-      atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);
+      if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
+        atomicAdd(hint + 1, 1u);
+        atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);
+        known_unit = b * p.Hkv + kvh;
+      }
     }
   }
 }
