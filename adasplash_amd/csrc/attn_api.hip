@@ -260,9 +260,9 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
     if (!workspace || workspace_bytes < w.total || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
     unsigned char* ws = (unsigned char*)workspace;
     p.vt = workspace;
-    // Sparse-support kernel first (alpha 1.5 / 2 behind the histogram entry point, no tile statistics asked for): it
-    // serves the row blocks whose supports are short and flags the others for the kernel below.
-    const bool sparse = w.slots > 0 && use_hist && (am == ATT_15 || am == ATT_2) && !tile_counts &&
+    // Sparse-support kernel first (alpha 1.5 / 2, either entry point, no tile statistics asked for): it serves the
+    // row blocks whose supports are short and flags the others for the kernel below.
+    const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && !tile_counts &&
                         (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
     if (sparse) {
       p.queue = (uint32_t*)(ws + w.queue_off);
