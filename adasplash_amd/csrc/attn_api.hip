@@ -241,6 +241,12 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.Npad = npad_of(N);
   p.n_mblk = mblocks_of(N);
   p.mask_words = mask_words_of(N);
+  // fp32 takes the reference's extra update: its solver makes `niter` refinements and one more behind the mask pass
+  // (adasplash/adasplash_v2.py:567-611 and :617-681), which is what brings the default niter = 1 to 1e-4.  The second
+  // and later steps run on the candidate lists of the list-carrying instance when they fit, without another K walk.
+  // The 16-bit types stop at `niter` steps (their tolerance is met with one) or take the sparse-support path, which
+  // converges fully.
+  if (dtype == ADSP_F32) niter += 1;
   p.niter = niter;
   p.causal = is_causal ? 1 : 0;
   p.use_hist = use_hist;
