@@ -27,6 +27,8 @@ _SIGNATURES = {
     "adsp_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "adsp_attn_bmask_words": (_sz, [_i]),
     "adsp_attn_v2_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "adsp_attn_v2_fwd_noalloc_max_bytes": (_sz, []),
+    "adsp_attn_v2_fwd_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "adsp_attn_v1_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _dbl, _i, _i, _vp, _sz,
                               _vp, _vp]),
     "adsp_attn_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),

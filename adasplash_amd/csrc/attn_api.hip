@@ -312,6 +312,48 @@ extern "C" int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, voi
                            workspace, workspace_bytes, nullptr, (hipStream_t)stream);
 }
 
+// ---- the entry point that allocates nothing -------------------------------------------------------------------
+namespace adsp {
+// Same work as adsp_attn_v2_fwd with the workspace taken from a file-scope device array instead of the caller.
+// `noalloc_scratch` is a host-side stand-in for the symbol here: the address the kernels can use is looked up once
+// per device with hipGetSymbolAddress (every GPU holds its own copy of the array) and only that pointer is passed on.
+constexpr size_t kNoAllocScratchBytes = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char noalloc_scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_noalloc_ptr[kMaxDevices] = {};
+
+static int noalloc_scratch_ptr(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return ADSP_ERR_LAUNCH;
+  void* ptr = __atomic_load_n(&g_noalloc_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!ptr) {
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(noalloc_scratch)) != hipSuccess || !ptr) return ADSP_ERR_LAUNCH;
+    __atomic_store_n(&g_noalloc_ptr[dev], ptr, __ATOMIC_RELEASE);  // (two threads racing here store the same address)
+  }
+  *out = ptr;
+  return ADSP_OK;
+}
+}  // namespace adsp
+
+extern "C" size_t adsp_attn_v2_fwd_noalloc_max_bytes(void) { return adsp::kNoAllocScratchBytes; }
+
+extern "C" int adsp_attn_v2_fwd_noalloc(const void* q, const void* k, const void* v, void* out, float* taus,
+                                        int32_t* bmask, const void* varlen, int varlen_bits, int B, int Hq, int Hkv,
+                                        int N, int D, int dtype, int niter, void* stream) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0) return ADSP_ERR_SHAPE;
+  if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return ADSP_ERR_SHAPE;
+  if (dtype != ADSP_F32 && dtype != ADSP_BF16 && dtype != ADSP_F16) return ADSP_ERR_DTYPE;
+  const size_t need = adsp_attn_workspace_bytes(B, Hq, Hkv, N, D, dtype);
+  if (need > adsp::kNoAllocScratchBytes) return ADSP_ERR_TOO_LARGE;
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = adsp::noalloc_scratch_ptr(&ws);
+    if (rc != ADSP_OK) return rc;
+  }
+  return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, Hq, Hkv, N, D, dtype, 1.5, 1, niter, 1, ws,
+                           need, nullptr, (hipStream_t)stream);
+}
+
 extern "C" int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
                                 const void* varlen, int varlen_bits, int B, int H, int N, int D, int dtype, double alpha,
                                 int is_causal, int niter, void* workspace, size_t workspace_bytes,
@@ -410,6 +452,7 @@ extern "C" const char* adsp_status_string(int status) {
     case ADSP_ERR_UNSUPPORTED: return "unsupported parameter combination";
     case ADSP_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case ADSP_ERR_LAUNCH: return "HIP launch failed";
+    case ADSP_ERR_TOO_LARGE: return "problem needs more scratch than the allocation-free entry point holds";
   }
   return "unknown status";
 }

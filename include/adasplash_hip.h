@@ -40,7 +40,8 @@ typedef enum {
   ADSP_ERR_ALIGN = 4,       /* a tensor base pointer is not 16-byte aligned */
   ADSP_ERR_UNSUPPORTED = 5, /* parameter combination the kernels do not implement */
   ADSP_ERR_WORKSPACE = 6,   /* workspace missing or smaller than adsp_attn_workspace_bytes() */
-  ADSP_ERR_LAUNCH = 7       /* the HIP runtime refused a launch (hipGetLastError() != success) */
+  ADSP_ERR_LAUNCH = 7,      /* the HIP runtime refused a launch (hipGetLastError() != success) */
+  ADSP_ERR_TOO_LARGE = 8    /* adsp_attn_v2_fwd_noalloc: the problem needs more scratch than the library holds */
 } adsp_status;
 
 /* Element types of q/k/v/out and x/y. */
@@ -103,6 +104,21 @@ size_t adsp_attn_bmask_words(int N);
 int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
                      const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
                      int niter, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * adsp_attn_v2_fwd without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * scratch memory (key-major copy of V, control words, flags and candidate streams of the sparse-support kernel)
+ * lives in a device array inside the library, 64 MiB on every GPU the library runs on, held until the process ends;
+ * problems whose adsp_attn_workspace_bytes() exceeds adsp_attn_v2_fwd_noalloc_max_bytes() are rejected with
+ * ADSP_ERR_TOO_LARGE.  The call allocates and frees nothing and records no memset (the kernels clear what must start
+ * at zero).  All calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race
+ * and must be serialised by the caller.  Other arguments, results and status codes as adsp_attn_v2_fwd.
+ */
+size_t adsp_attn_v2_fwd_noalloc_max_bytes(void);
+int adsp_attn_v2_fwd_noalloc(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                             const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
+                             int niter, void* stream);
 
 /*
  * AdaSplash-1 (block-mask) forward: alpha-entmax attention for any alpha in (1, 2], causal or not,
