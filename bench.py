@@ -12,7 +12,9 @@ Workloads (``--workload``):
   c2   entmax rows x[16384, 8192] = 4*N(0,1), bf16 and fp32, alpha in {1.5, 2}
   c2_bwd  entmax rows backward on the same shape (reads y, writes dx, reads dy on the support only)
   c4_bwd, c3_bwd   dq, dk, dv of the c4 / c3 forward (2.5 x its dense-equivalent FLOPs per step)
-The default run also times the entmax rows workloads (c2, c2_bwd) and the c4 backward and reports them under ``extra``.
+The default run also times c3, c5, the entmax rows workloads (c2, c2_bwd) and the c4 backward and reports them under
+``extra``, with the v2 tile statistics of the headline workload (key tiles of 128 rows x 64 keys inside the causal /
+valid domain, those the block mask keeps, and the share of row blocks the sparse-support kernel served).
 
 Dense-equivalent FLOPs of causal attention = 2 * Hq * D * sum_b L_b^2 (QK^T and PV, each halved by
 causality); non-causal = 4 * B * H * N^2 * D.  Rows bytes = rows * cols * (sizeof(in) + sizeof(out)).
@@ -36,6 +38,15 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_HBM_TRAFFIC_BYTES = {"c4": 1.511e9, "c3": 0.1998e9, "c5": 0.632e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5373e9,
                               "c2_bwd_f32": 1.0848e9, "c2_bwd_bf16": 0.5476e9,
                               "c4_bwd": 23.57e9}  # c4_bwd: dq kernel 2.03e9 + dk/dv kernel 21.54e9
+
+
+# The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
+# probe of the score distribution, the sparse-support kernel, the key-major copy of V and the dense kernel, of which
+# the last two return at once unless the sparse-support kernel left row blocks over (c3: the probe marks every head
+# dense and the dense kernel does all the work).
+FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + this + V copy and attn_fwd_kernel on leftovers)",
+               "c3": "attn_fwd_kernel<bf16, 64, single step> (step = probe + sparse-support kernel stepping aside + V copy + this)",
+               "c5": "attn_fwd_kernel<bf16, 64, generic alpha, candidate lists>"}
 
 
 def _events_ms(fn, steps, warmup):
@@ -91,6 +102,33 @@ def make_c5(device, seed=42):
     return (q, k, v), flops, cfg
 
 
+def v2_tile_stats(q, k, v, varlen):
+    """Tile statistics of one adasplash_v2 forward, from the block mask it writes: a tile is 128 query rows x 64 keys.
+    `grid` counts all tiles of the padded problem, `domain` those that hold a valid (row, key) pair under the causal
+    mask and the sequence lengths (the difference is excluded by causality or padding, not by tau), `kept` those in
+    which some row has a non-zero probability; `skipped_by_tau` = domain - kept."""
+    from adasplash_amd import _attention
+
+    B, Hq, N, _ = q.shape
+    _, _, bmask = _attention.launch_forward(q, k, v, version=2, alpha=1.5, is_causal=True, niter=1, varlen=varlen)
+    n_blk, n_tile = (N + 127) // 128, (N + 63) // 64
+    lens = varlen.cpu().long() if varlen is not None else torch.full((B,), N, dtype=torch.long)
+    m0 = torch.arange(n_blk) * 128
+    row_hi = torch.minimum(m0[None, :] + 128, lens[:, None])  # [B, n_blk]
+    domain_per_blk = torch.where(m0[None, :] < lens[:, None], (row_hi + 63) // 64, torch.zeros_like(row_hi))
+    domain = int(domain_per_blk.sum()) * Hq
+    words = bmask.view(B, Hq, n_blk, -1).cpu()
+    kept = 0
+    for w in range(words.shape[-1]):
+        x = words[..., w].to(torch.int64) & 0xFFFFFFFF
+        for bit in range(32):
+            kept += int(((x >> bit) & 1).sum())
+    grid = B * Hq * n_blk * n_tile
+    return {"tile": "128 rows x 64 keys", "tiles_grid": grid, "tiles_domain": domain, "tiles_kept": kept,
+            "tiles_excluded_by_causality_or_padding": grid - domain, "tiles_skipped_by_tau": domain - kept,
+            "tiles_skipped_frac_of_domain": (domain - kept) / domain if domain else None}
+
+
 def bench_attention(name, steps, warmup, device, backward=False):
     import adasplash_amd as A
 
@@ -120,6 +158,8 @@ def bench_attention(name, steps, warmup, device, backward=False):
     tflops = flops / (ms * 1e-3) / 1e12
     res = {"ms_per_step": ms, "wall_ms_per_step": wall_ms, "eff_tflops": tflops, "flops_per_step": flops,
            "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS, "config": cfg}
+    if name in ("c4", "c3") and not backward:
+        res["tiles"] = v2_tile_stats(q, k, v, varlen)
     if name == "c5":
         from adasplash_amd.adasplash_block_mask import tile_sparsity
 
@@ -248,8 +288,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    from adasplash_amd import _lib
+
     line = {"metric": "v2 fwd ms + eff. TFLOPS/%MFMA peak (N=8192,D=128,GQA); entmax rows GB/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+            "build_id": _lib.build_id(), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "data": "synthetic"}
     if args.workload == "copy":
         # plain device copy of known size: the reference point for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE
@@ -286,15 +328,23 @@ def main():
                      "roofline": {"bound": "mfma", "achieved": res["eff_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                                   "unit": "TFLOP/s", "frac": res["frac_mfma_peak"],
                                   "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
-                                  "kernel": "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel" if bwd else "attn_fwd_kernel",
+                                  "kernel": "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel" if bwd else FWD_KERNELS[args.workload],
                                   "flops_per_launch": res["flops_per_step"]},
                      "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k == "wall_ms_per_step"}})
+        if "tiles" in res:
+            line["tiles"] = res["tiles"]
         if not args.no_extra:
             del res
             torch.cuda.empty_cache()
             line["extra"]["entmax_rows"] = bench_rows(args.steps, args.warmup, device)
             line["extra"]["entmax_rows_backward"] = bench_rows_backward(args.steps, args.warmup, device)
             if args.workload == "c4":
+                for other in ("c3", "c5"):
+                    r = bench_attention(other, args.steps, args.warmup, device)
+                    line["extra"][other] = {k: r[k] for k in r if k != "wall_ms_per_step"}
+                    line["extra"][other]["kernel"] = FWD_KERNELS[other]
+                    del r
+                    torch.cuda.empty_cache()
                 b = bench_attention("c4", max(3, args.steps // 2), 1, device, backward=True)
                 line["extra"]["attention_backward"] = {k: b[k] for k in ("ms_per_step", "eff_tflops", "frac_mfma_peak",
                                                                          "flops_per_step")}
