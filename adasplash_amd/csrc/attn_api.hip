@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
 // Workspace of the forward for the 16-bit types: the key-major copy of V, then -- for the head dims the
 // sparse-support kernel serves -- its work counters, its per-row-block flags and its candidate streams.
 constexpr int kSparseMaxSlots = 1024;                       // workgroups of the persistent kernel
-constexpr size_t kSparseSlotBytes = (size_t)4 * 1472 * 8;   // four waves x 1472 candidates x (score, key)
+constexpr size_t kSparseSlotBytes = (size_t)4 * 1616 * 8;   // four waves x 1616 candidates x (score, key)
 struct FwdWorkspace {
   size_t vt_bytes, queue_off, flags_off, events_off, total;
   int slots;  // 0: no sparse-support kernel for these dimensions
@@ -191,7 +191,7 @@ static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
   if (dtype == ADSP_F32) return w;
   w.vt_bytes = (size_t)B * Hkv * D * npad_of(N) * 2;
   w.total = w.vt_bytes;
-  if (D == 64 || D == 128) {
+  if ((D == 64 || D == 128) && N <= 65536) {  // (the candidate lists hold 16-bit key indices)
     const long long items = (long long)B * Hq * mblocks_of(N);
     long long slots = (items + 7) / 8 * 8;
     if (slots > kSparseMaxSlots) slots = kSparseMaxSlots;

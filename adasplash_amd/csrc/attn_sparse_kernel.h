@@ -28,9 +28,10 @@
 namespace adsp {
 
 #ifndef ADSP_SPARSE_WAVES
-#define ADSP_SPARSE_WAVES 3
+#define ADSP_SPARSE_WAVES 4
 #endif
-constexpr int kSparseStreamCap = 1472;  // candidates per wave (what SparseGeo::kListCap may be at most)
+constexpr int kSparseStreamCap = 1616;  // candidates per wave the workspace slot holds (SparseGeo::kListCap is at most this)
+constexpr int kSparseMaxKeys = 65536;   // the lists hold 16-bit key indices
 
 // acc[2 i] += v[i].lo * p, acc[2 i + 1] += v[i].hi * p for the eight elements of a 16-byte chunk, with the weight given
 // as the pairs plo = (p, 0) and phi = (0, p) of the element type: eight two-term dot products with fp32 accumulation.
@@ -68,15 +69,17 @@ template <typename T, int D> struct SparseGeo {
   static constexpr int kNW = 4;
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
-  // two K stages during the walks; afterwards the whole array holds the candidate lists, then the output staging
-  static constexpr int kLds = 2 * G::kKTile > 48 * 1024 ? 2 * G::kKTile : 48 * 1024;
+  // Four workgroups share a CU (one wave of each per SIMD): 40 KB of LDS each.  Two K stages during the walks, with
+  // the waves' event rings behind them; afterwards the whole array holds the candidate lists.
+  static constexpr int kLds = 2 * G::kKTile + 4096 > 39 * 1024 ? 2 * G::kKTile + 4096 : 39 * 1024;  // (1 KB left for the small arrays)
   static constexpr int kWaveLds = kLds / kNW;
-  static constexpr int kListCap = (kWaveLds - 512) / 8;  // candidates per wave: the lists, then the rows' counters
-  // during walk 2 the LDS behind the two K stages holds a ring of events per wave
+  // candidates per wave: scores (fp32) and keys (16 bits: the path serves up to 65536 keys) in two arrays, then the
+  // rows' counters, offsets and 1 / sum
+  static constexpr int kListCapRaw = (kWaveLds - 512) / 6 / 8 * 8;
+  static constexpr int kListCap = kListCapRaw > kSparseStreamCap ? kSparseStreamCap : kListCapRaw;
   static constexpr int kRingBytes = (kLds - 2 * G::kKTile) / kNW;
   static constexpr int kRing = kRingBytes / 36 > 192 ? 192 : kRingBytes / 36;  // events: 8 scores and a tag
-  static_assert(kRing >= 64, "a half block can bring 64 events");
-  static_assert(kListCap <= kSparseStreamCap, "the workspace slot holds kSparseStreamCap candidates per wave");
+  static_assert(kRing >= 32, "half a wave can bring 32 events at once");
 };
 
 template <typename T, int D, int AM>
@@ -386,7 +389,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
     float* const ring = reinterpret_cast<float*>(lds_all + 2 * G::kKTile + wave * SG::kRingBytes);
     uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
-    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)SG::kListCap;
+    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
     int ring_n = 0, stream_n = 0;  // wave-uniform
     // (kt: the tile being worked on; a stream that fills faster than the tiles go by will not last: give up early)
     auto flush = [&](int parity, int kt) {
@@ -425,20 +428,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
       ring_n = 0;
     };
+    // the lanes of `m` (those of them for which `mine` holds put their half block) take consecutive ring slots
+    auto put = [&](unsigned long long m, bool mine, const f32x16& s, int first, uint32_t tag, int kt) {
+      const int c = __builtin_popcountll(m);
+      if (ring_n + c > SG::kRing) flush(kt & 1, kt);
+      if (mine) {
+        const int slot = ring_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        f32x4 w0 = {s[first], s[first + 1], s[first + 2], s[first + 3]};
+        f32x4 w1 = {s[first + 4], s[first + 5], s[first + 6], s[first + 7]};
+        *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
+        *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
+        ring_tag[slot] = (tag << 6) | (uint32_t)lane;
+      }
+      ring_n += c;
+    };
     auto collect = [&](const f32x16& s, int first, float hmax, uint32_t tag, int kt) {
       const unsigned long long m = __builtin_amdgcn_ballot_w64(hmax > 0.f);
       if (m != 0ull) {
-        const int c = __builtin_popcountll(m);
-        if (ring_n + c > SG::kRing) flush(kt & 1, kt);
-        if (hmax > 0.f) {
-          const int slot = ring_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-          f32x4 w0 = {s[first], s[first + 1], s[first + 2], s[first + 3]};
-          f32x4 w1 = {s[first + 4], s[first + 5], s[first + 6], s[first + 7]};
-          *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
-          *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
-          ring_tag[slot] = (tag << 6) | (uint32_t)lane;
+        if (__builtin_popcountll(m) <= SG::kRing) {
+          put(m, hmax > 0.f, s, first, tag, kt);
+        } else {  // more events than the ring holds at once (the first tiles of a sequence): in two halves
+          put(m & 0xffffffffull, hmax > 0.f && lane < 32, s, first, tag, kt);
+          put(m & ~0xffffffffull, hmax > 0.f && lane >= 32, s, first, tag, kt);
         }
-        ring_n += c;
       }
     };
     walk([&](int kt, const unsigned char* kt_lds) {
@@ -472,8 +484,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 
     // ---- the wave's stream -> per-row lists in its share of LDS (a counting sort by row) ----------------------------
     unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
-    uint2* const lst = reinterpret_cast<uint2*>(wave_lds);                                   // kListCap entries
-    uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 8);     // 32 counters
+    float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap scores, later probabilities
+    uint16_t* const lkey = reinterpret_cast<uint16_t*>(wave_lds + SG::kListCap * 4);         // their keys
+    uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 6);     // 32 counters
     uint32_t* const row_start = row_cnt + 32;                                                // 33 offsets
     float* const row_inv = reinterpret_cast<float*>(row_start + 33);                         // 32 x 1 / sum p
     if (lane < 32) row_cnt[lane] = 0u;
@@ -502,7 +515,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 #pragma unroll
       for (int j = 0; j < kPer; ++j) {
         const int e = j * 64 + lane;
-        if (e < stream_n) lst[row_start[(ent[j].y >> 20) & 31u] + pos[j]] = uint2{ent[j].x, ent[j].y & 0xfffffu};
+        if (e < stream_n) {
+          const uint32_t at = row_start[(ent[j].y >> 20) & 31u] + pos[j];
+          lval[at] = __builtin_bit_cast(float, ent[j].x);
+          lkey[at] = (uint16_t)(ent[j].y & 0xffffu);
+        }
       }
     }
 
@@ -514,7 +531,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       for (int it = 0; it < 24; ++it) {
         float a0 = 0.f, a1 = 0.f;
         for (int e = row_lo + lh; e < row_end; e += 2) {
-          const float u = fmaxf(__builtin_bit_cast(float, lst[e].x) - t, 0.f);
+          const float u = fmaxf(lval[e] - t, 0.f);
           if constexpr (AM == ATT_15) {
             a0 = fmaf(u, u, a0);
             a1 += u;
@@ -538,11 +555,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       int w = row_lo;
       if (lh == 0) {
         for (int e = row_lo; e < row_end; ++e) {
-          const uint2 en = lst[e];
-          const float u = __builtin_bit_cast(float, en.x) - t;
+          const float u = lval[e] - t;
+          const uint16_t key = lkey[e];
           if (u > 0.f) {
             const float pv = (AM == ATT_15) ? u * u : u;
-            lst[w] = uint2{__builtin_bit_cast(uint32_t, pv), en.y};
+            lval[w] = pv;
+            lkey[w] = key;
             ++w;
             psum += pv;
           }
@@ -578,10 +596,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
             pw[j] = 0u;
             vv[j] = u32x4{0u, 0u, 0u, 0u};
             if (eb + j < e_hi) {
-              const uint2 en = lst[eb + j];
-              pw[j] = en.x;
-              vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)en.y * (D * 2));
-              if (col == 0) atomicOr(&mask_out[(en.y / kBN) >> 5], 1u << ((en.y / kBN) & 31));
+              const uint32_t key = lkey[eb + j];
+              pw[j] = __builtin_bit_cast(uint32_t, lval[eb + j]);
+              vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
+              if (col == 0) atomicOr(&mask_out[(key / kBN) >> 5], 1u << ((key / kBN) & 31));
             }
           }
 #pragma unroll

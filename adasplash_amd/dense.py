@@ -15,12 +15,13 @@ import torch
 
 
 def _varlen_mask(varlen, size, padding):
-    positions = torch.arange(size, device=varlen.device)
-    if padding == "right":
-        return positions[None, :] < varlen[:, None]
-    if padding == "left":
-        return positions[None, :] >= size - varlen[:, None]
-    raise ValueError("padding must be either 'right' or 'left'.")
+    """(B, size) boolean map of the positions inside each sequence: the first ``varlen[b]`` of them with right
+    padding, the last ``varlen[b]`` with left padding."""
+    if padding not in ("right", "left"):
+        raise ValueError("padding must be either 'right' or 'left'.")
+    first = torch.zeros_like(varlen) if padding == "right" else size - varlen
+    idx = torch.arange(size, device=varlen.device).unsqueeze(0)
+    return (idx >= first.unsqueeze(1)) & (idx < (first + varlen).unsqueeze(1))
 
 
 def _alibi_bias(q, k, alibi_slopes):
@@ -58,7 +59,9 @@ def slow_entmax_attention(q, k, v, alpha=1.5, varlen=None, is_causal=False, padd
 
     dev = q.device
     q_len, k_len, head_dim = q.shape[2], k.shape[2], q.shape[3]
-    scores = torch.matmul(q, k.transpose(-1, -2)) * (1.0 / math.sqrt(head_dim))
+    # the score matrix is formed and kept in fp32 whatever the input type (a 16-bit GEMM result would round scores of
+    # a few units by up to 2^-8 of their size before the entmax, which the fused kernels never do)
+    scores = torch.matmul(q.float(), k.float().transpose(-1, -2)) * (1.0 / math.sqrt(head_dim))
     if alibi_slopes is not None:
         scores = scores + _alibi_bias(q, k, alibi_slopes)
 
@@ -80,7 +83,7 @@ def slow_entmax_attention(q, k, v, alpha=1.5, varlen=None, is_causal=False, padd
         scores = scores.masked_fill(~rows_live, 0.0)  # padded rows stay finite here and are zeroed below
 
     probs = triton_entmax(scores.contiguous(), alpha=alpha, n_iter=niter, fast_math=False)
-    # fp32 slopes promote 16-bit scores to fp32; the probabilities go back to v's type for the second product
+    # the probabilities go back to v's type for the second product
     out = torch.matmul(probs.to(v.dtype), v)
     return out if rows_live is None else out.masked_fill(~rows_live, 0)
 

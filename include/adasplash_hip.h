@@ -82,7 +82,7 @@ int adsp_entmax_rows_bwd(const void* y, const void* dy, void* dx, int64_t rows, 
 /*
  * Bytes of scratch the forward entry points need for these dimensions; 0 for fp32.  For the 16-bit types: a
  * key-major copy of V and, at head dims 64 and 128, the work counters, row-block flags and event slots of the
- * sparse-support kernel (up to 1024 slots of 46 KiB).  The buffer must be 16-byte aligned device memory; its
+ * sparse-support kernel (up to 1024 slots of 51 KiB; sequences of up to 65536 keys).  The buffer must be 16-byte aligned device memory; its
  * contents need not survive between calls.  For the block-mask variant pass Hq = Hkv = H.
  */
 size_t adsp_attn_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);

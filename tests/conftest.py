@@ -29,3 +29,21 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def golden_dir():
     return ROOT / "tests" / "golden"
+
+
+def pytest_terminal_summary(terminalreporter):
+    """16-bit parity figures of the run: the raw max-abs error beside the magnitude-scaled one the assertions use."""
+    try:
+        from tests import gpu_util
+    except Exception:  # noqa: BLE001
+        return
+    rec = gpu_util.RAW_16BIT
+    if not rec:
+        return
+    worst_raw = max(rec, key=lambda r: r[0])
+    worst_small = max(rec, key=lambda r: r[1])
+    worst_scaled = max(rec, key=lambda r: r[2])
+    terminalreporter.write_line(
+        f"16-bit comparisons: {len(rec)}; worst raw max-abs {worst_raw[0]:.3e} (where max |want| = {worst_raw[3]:.2f}); "
+        f"worst raw max-abs over entries with |want| <= 2: {worst_small[1]:.3e}; worst magnitude-scaled: "
+        f"{worst_scaled[2]:.3e}")

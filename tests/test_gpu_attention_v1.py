@@ -228,3 +228,22 @@ def test_output_from_lists_matches_output_walk():
     assert max_err(walked.cpu(), gathered.cpu().double()) < 2e-2  # one bf16 step: the walk rounds P to bf16 before its PV product
     want = exact.dense_entmax_attention(q.cpu(), k.cpu(), v.cpu(), 1.333, False, varlen=varlen.cpu())
     assert max_err(gathered.cpu(), want) < 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("alpha,causal", [(1.5, False), (1.5, True), (1.333, False), (2.0, True)])
+def test_no_block_mask_name_is_served_by_the_same_kernels(dtype, alpha, causal):
+    """``adasplash_no_block_mask`` (adasplash/__init__.py:33-36, kernel file adasplash/adasplash_no_block_mask.py)
+    computes the same function without the block mask; here the name is served by the block-mask kernels.  Parity
+    against the dense oracle with and without variable lengths."""
+    torch.manual_seed(3)
+    q, k, v = (torch.randn(2, 2, 320, 64).to(dtype) for _ in range(3))
+    tol = tol_for(dtype, alpha)
+    out = A.adasplash_no_block_mask(q.to(DEV), k.to(DEV), v.to(DEV), alpha=alpha, is_causal=causal)
+    assert out.dtype == dtype
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, alpha, causal)) < tol
+    varlen = torch.tensor([320, 131], dtype=torch.int32)
+    out = A.adasplash_no_block_mask(q.to(DEV), k.to(DEV), v.to(DEV), alpha=alpha, is_causal=causal,
+                                    varlen=varlen.to(DEV))
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, alpha, causal, varlen)) < tol
+    assert (out[1, :, 131:] == 0).all()

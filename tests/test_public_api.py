@@ -165,7 +165,7 @@ def test_sizing_helpers_and_status_strings():
     assert lib.adsp_attn_workspace_bytes(2, 2, 2, 100, 32, _lib.ADSP_F16) == 2 * 2 * 32 * 128 * 2
     # ... and at head dims 64 / 128 the sparse-support kernel's counters, flags and candidate slots (at most 1024)
     vt = 8 * 8 * 128 * 8192 * 2
-    slot = 4 * 1472 * 8
+    slot = 4 * 1616 * 8
     assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) == vt + 256 + 768 + 8 * 32 * 64 * 4 + 1024 * slot  # (8 * 8 + 1) hint pairs, padded to 256
     small = lib.adsp_attn_workspace_bytes(1, 2, 2, 128, 64, _lib.ADSP_F16)
     assert 8 * slot < small < 8 * slot + 2 * 64 * 128 * 2 + 1024
