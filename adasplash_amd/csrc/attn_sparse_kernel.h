@@ -27,8 +27,14 @@
 
 namespace adsp {
 
+#ifndef ADSP_GATHER_DEPTH
+#define ADSP_GATHER_DEPTH 8
+#endif
+#ifndef ADSP_SPARSE_STAGES
+#define ADSP_SPARSE_STAGES 2
+#endif
 #ifndef ADSP_SPARSE_WAVES
-#define ADSP_SPARSE_WAVES 4
+#define ADSP_SPARSE_WAVES (ADSP_SPARSE_STAGES == 2 ? 4 : 3)
 #endif
 constexpr int kSparseStreamCap = 1616;  // candidates per wave the workspace slot holds (SparseGeo::kListCap is at most this)
 constexpr int kSparseMaxKeys = 65536;   // the lists hold 16-bit key indices
@@ -69,15 +75,18 @@ template <typename T, int D> struct SparseGeo {
   static constexpr int kNW = 4;
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
-  // Four workgroups share a CU (one wave of each per SIMD): 40 KB of LDS each.  Two K stages during the walks, with
-  // the waves' event rings behind them; afterwards the whole array holds the candidate lists.
-  static constexpr int kLds = 2 * G::kKTile + 4096 > 39 * 1024 ? 2 * G::kKTile + 4096 : 39 * 1024;  // (1 KB left for the small arrays)
+  // K stages during the walks, with the waves' event rings behind them; afterwards the whole array holds the
+  // candidate lists.  Two stages: 39 KB, four workgroups per CU (one wave of each per SIMD); three stages (a tile
+  // load has two tile times to arrive): 52 KB at head dim 128, three workgroups per CU.
+  static constexpr int kStages = ADSP_SPARSE_STAGES;
+  static constexpr int kMinLds = kStages == 2 ? 39 * 1024 : 52 * 1024;  // (1 KB left for the small arrays)
+  static constexpr int kLds = kStages * G::kKTile + 4608 > kMinLds ? kStages * G::kKTile + 4608 : kMinLds;  // rings of >= 32 events
   static constexpr int kWaveLds = kLds / kNW;
   // candidates per wave: scores (fp32) and keys (16 bits: the path serves up to 65536 keys) in two arrays, then the
   // rows' counters, offsets and 1 / sum
   static constexpr int kListCapRaw = (kWaveLds - 512) / 6 / 8 * 8;
   static constexpr int kListCap = kListCapRaw > kSparseStreamCap ? kSparseStreamCap : kListCapRaw;
-  static constexpr int kRingBytes = (kLds - 2 * G::kKTile) / kNW;
+  static constexpr int kRingBytes = (kLds - kStages * G::kKTile) / kNW;
   static constexpr int kRing = kRingBytes / 36 > 192 ? 192 : kRingBytes / 36;  // events: 8 scores and a tag
   static_assert(kRing >= 32, "half a wave can bring 32 events at once");
 };
@@ -96,8 +105,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   // parity and read the other one behind the next barrier, so no wave can read a word another one is still setting
   __shared__ uint32_t s_giveup[2];
   extern __shared__ uint32_t mask_out[];  // p.mask_words words: key tiles that hold a non-zero probability
-  unsigned char* const k_lds0 = lds_all;
-  unsigned char* const k_lds1 = lds_all + G::kKTile;
 
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int N = p.N;
@@ -248,26 +255,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
     };
-    // body(kt, tile) over all key tiles of the row block, K double-buffered; stops when a lane gave up
+    // body(kt, tile) over all key tiles of the row block; stops when a lane gave up.  The K tiles go through a ring of
+    // kStages LDS buffers: the load of tile t + kStages - 1 is issued behind the barrier that opens tile t (every wave
+    // is done with tile t - 1, whose buffer it takes) and has kStages - 1 tile times to arrive.
     auto walk = [&](auto&& body) {
+      constexpr int kStages = SG::kStages;
       __syncthreads();
-      int cur = 0;
-      issue_k(k_lds0, 0);
-      for (;;) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+#pragma unroll
+      for (int s = 0; s < kStages - 1; ++s)
+        if (s < nt) issue_k(lds_all + s * G::kKTile, s);
+      int stage = 0;  // buffer of tile cur
+      for (int cur = 0; cur < nt; ++cur) {
+        // this wave's share of tile cur has landed: everything but the loads issued after it (those of the tiles in
+        // between; stores issued after it only make the wait longer than needed)
+        if (cur + kStages - 1 <= nt) {
+          if constexpr (kStages == 2) __builtin_amdgcn_s_waitcnt(0x0f70);
+          else __builtin_amdgcn_s_waitcnt(0x0f70 | ((kStages - 2) * kKPer));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);  // the last tiles: nothing was issued behind them
+        }
         __syncthreads();
         if (s_giveup[(cur + 1) & 1]) break;  // set while the previous tile was worked on
-        if (cur + 1 < nt) issue_k(k_lds1, cur + 1);
+        const int pre = cur + kStages - 1;
+        if (pre < nt) issue_k(lds_all + (stage == 0 ? kStages - 1 : stage - 1) * G::kKTile, pre);
         __builtin_amdgcn_sched_barrier(0);
-        body(cur, k_lds0);
-        if (++cur >= nt) break;
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-        __syncthreads();
-        if (s_giveup[(cur + 1) & 1]) break;
-        if (cur + 1 < nt) issue_k(k_lds0, cur + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        body(cur, k_lds1);
-        if (++cur >= nt) break;
+        body(cur, lds_all + stage * G::kKTile);
+        stage = stage + 1 == kStages ? 0 : stage + 1;
       }
     };
     // S^T of one tile (two 32-key blocks), accumulators preloaded with `init`; f(s0, s1) unless no row of the wave
@@ -387,7 +400,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // ring in LDS (slots are handed out with a ballot: no atomics).  When the ring is full the wave empties it, one
     // event per lane: the positive entries go to the wave's candidate stream in global memory as (score - lo, key and
     // row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
-    float* const ring = reinterpret_cast<float*>(lds_all + 2 * G::kKTile + wave * SG::kRingBytes);
+    float* const ring = reinterpret_cast<float*>(lds_all + SG::kStages * G::kKTile + wave * SG::kRingBytes);
     uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
     uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
     int ring_n = 0, stream_n = 0;  // wave-uniform
@@ -578,7 +591,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     {
       constexpr int kLPR = D / 8;         // lanes per row
       constexpr int kGroups = 64 / kLPR;  // rows in progress per wave
-      constexpr int kDepth = 8;
+      constexpr int kDepth = ADSP_GATHER_DEPTH;
       const int grp = lane / kLPR, col = lane % kLPR;
       const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
       unsigned char* obase = reinterpret_cast<unsigned char*>(p.out) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
