@@ -532,6 +532,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           const uint32_t at = row_start[(ent[j].y >> 20) & 31u] + pos[j];
           lval[at] = __builtin_bit_cast(float, ent[j].x);
           lkey[at] = (uint16_t)(ent[j].y & 0xffffu);
+          // the tile mask takes every candidate's tile: a superset of the tiles with a non-zero probability by the few
+          // candidates below the threshold, cheaper to mark here (one entry per lane) than in the output loop
+          const uint32_t tile = (ent[j].y & 0xffffu) / kBN;
+          atomicOr(&mask_out[tile >> 5], 1u << (tile & 31));
         }
       }
     }
@@ -572,7 +576,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           const uint16_t key = lkey[e];
           if (u > 0.f) {
             const float pv = (AM == ATT_15) ? u * u : u;
-            lval[w] = pv;
+            lval[w] = __builtin_bit_cast(float, pack2<T>(pv, 0.f));  // the pair (p, 0) of the element type, as the output loop takes it
             lkey[w] = key;
             ++w;
             psum += pv;
@@ -612,13 +616,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
               const uint32_t key = lkey[eb + j];
               pw[j] = __builtin_bit_cast(uint32_t, lval[eb + j]);
               vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
-              if (col == 0) atomicOr(&mask_out[(key / kBN) >> 5], 1u << ((key / kBN) & 31));
             }
           }
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
-            const uint32_t plo = pack2<T>(__builtin_bit_cast(float, pw[j]), 0.f), phi = plo << 16;
-            dot2_chunk<T>(acc, vv[j], plo, phi);
+            dot2_chunk<T>(acc, vv[j], pw[j], pw[j] << 16);
           }
         }
         const float inv = row_inv[r];
