@@ -85,6 +85,31 @@ __global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restri
   }
 }
 
+// e4m3 copy of K for the first walk of the sparse-support forward: [B * Hkv][Npad][D] bytes in the order of K, values
+// beyond the format's range saturated, rows from N on zero.  A thread converts 16 values.  Heads the probe has marked
+// as dense are skipped (`hints`: two words per head).
+template <typename T>
+__global__ __launch_bounds__(256) void k8_layout_kernel(const uint16_t* __restrict__ k, unsigned char* __restrict__ k8, int N,
+                                                       int Npad, int D, const uint32_t* hints) {
+  const size_t head = blockIdx.y;
+  if (hints[2 * head] >= (1u << 20)) return;
+  const int per_row = D / 16;
+  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long long)Npad * per_row) return;
+  const int row = (int)(id / per_row), c = (int)(id % per_row);
+  u32x4 out = {0u, 0u, 0u, 0u};
+  if (row < N) {
+    const uint16_t* src = k + (head * (size_t)N + row) * D + c * 16;
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(src), hi = *reinterpret_cast<const u32x4*>(src + 8);
+#pragma unroll
+    for (int e = 0; e < 4; e += 2) {
+      out[e >> 1] = cvt_e4m3_pair(unpack_lo<T>(lo[e + 1]), unpack_hi<T>(lo[e + 1]), cvt_e4m3_pair(unpack_lo<T>(lo[e]), unpack_hi<T>(lo[e]), 0u, false), true);
+      out[2 + (e >> 1)] = cvt_e4m3_pair(unpack_lo<T>(hi[e + 1]), unpack_hi<T>(hi[e + 1]), cvt_e4m3_pair(unpack_lo<T>(hi[e]), unpack_hi<T>(hi[e]), 0u, false), true);
+    }
+  }
+  *reinterpret_cast<u32x4*>(k8 + (head * (size_t)Npad + row) * D + c * 16) = out;
+}
+
 static unsigned vt_layout_blocks(int Npad, int D) {  // 256 / D tiles of 64 keys per block
   const int tiles = Npad / kBN, per_block = 256 / D;
   return (unsigned)((tiles + per_block - 1) / per_block);
@@ -178,11 +203,12 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
 }
 
 // Workspace of the forward for the 16-bit types: the key-major copy of V, then -- for the head dims the
-// sparse-support kernel serves -- its work counters, its per-row-block flags and its candidate streams.
+// sparse-support kernel serves -- its work counters, its per-row-block flags, its candidate streams and the e4m3 copy
+// of K that its first walk reads.
 constexpr int kSparseMaxSlots = 1024;                       // workgroups of the persistent kernel
 constexpr size_t kSparseSlotBytes = (size_t)4 * 1616 * 8;   // four waves x 1616 candidates x (score, key)
 struct FwdWorkspace {
-  size_t vt_bytes, queue_off, flags_off, events_off, total;
+  size_t vt_bytes, queue_off, flags_off, events_off, k8_off, total;
   int slots;  // 0: no sparse-support kernel for these dimensions
 };
 static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
@@ -199,7 +225,8 @@ static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     w.queue_off = align256(w.vt_bytes);
     w.flags_off = align256(w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8);  // eight counters, then two hint words per K/V head and two more
     w.events_off = align256(w.flags_off + (size_t)items * 4);
-    w.total = w.events_off + (size_t)slots * kSparseSlotBytes;
+    w.k8_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
+    w.total = w.k8_off + (size_t)B * Hkv * npad_of(N) * D;  // the e4m3 copy of K
   }
   return w;
 }
@@ -259,6 +286,7 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.queue = nullptr;
   p.hints = nullptr;
   p.events = nullptr;
+  p.k8 = nullptr;
 
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
@@ -275,8 +303,15 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
       p.hints = p.queue + 64;
       p.block_flags = (int32_t*)(ws + w.flags_off);
       p.events = ws + w.events_off;
-      if (dtype == ADSP_BF16) hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
-      else hipLaunchKernelGGL(attn_probe_kernel<f16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
+      p.k8 = ws + w.k8_off;
+      const dim3 k8_grid((unsigned)(((long long)p.Npad * (D / 16) + 255) / 256), (unsigned)(B * Hkv));
+      if (dtype == ADSP_BF16) {
+        hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
+        hipLaunchKernelGGL(k8_layout_kernel<bf16_t>, k8_grid, dim3(256), 0, s, (const uint16_t*)k, ws + w.k8_off, N, p.Npad, D, (const uint32_t*)p.hints);
+      } else {
+        hipLaunchKernelGGL(attn_probe_kernel<f16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
+        hipLaunchKernelGGL(k8_layout_kernel<f16_t>, k8_grid, dim3(256), 0, s, (const uint16_t*)k, ws + w.k8_off, N, p.Npad, D, (const uint32_t*)p.hints);
+      }
       int rc = dtype == ADSP_BF16 ? (D == 64 ? launch_attn_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_sparse_bf16_d128(p, am, w.slots, s))
                                   : (D == 64 ? launch_attn_sparse_f16_d64(p, am, w.slots, s) : launch_attn_sparse_f16_d128(p, am, w.slots, s));
       if (rc != 0) return ADSP_ERR_LAUNCH;

@@ -41,6 +41,7 @@ struct AttnParams {
   uint32_t* queue;        // eight work counters, one per XCD, then the two control words above; zero at launch
   uint32_t* hints;        // [B * Hkv + 1][2] row blocks {given up, served} per K/V head, then over all heads; zero at launch
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
+  const unsigned char* k8;  // fp8 (e4m3) copy of K, [B * Hkv][Npad][D] bytes, rows past N zero: the operand of the first walk
 };
 
 }  // namespace adsp

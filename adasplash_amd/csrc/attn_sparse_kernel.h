@@ -5,10 +5,14 @@
 // output needs only those few keys.  This kernel finds them with two walks over K whose vector work per score is
 // about one instruction, then solves the threshold and forms the output from the short candidate lists:
 //
-//   walk 1  S^T = K Q^T per tile on MFMA; a lane keeps the four largest block maxima of its half of the row's keys.
-//           The threshold of any subset of a row's scores is a lower bound of the row's threshold (f only grows when
-//           entries are added), so a few Newton steps from the left on the row's eight kept values give a rigorous
-//           lower bound `lo` that lies within a few hundredths (in z) of the threshold for such rows.
+//   walk 1  S^T = K Q^T per tile on the fp8 MFMA (twice the 16-bit rate, half the tile bytes) from an e4m3 copy of K
+//           and Q fragments rounded the same way; a lane keeps the four largest block maxima of its half of the row's
+//           keys together with the keys they belong to (the key's position rides in the low mantissa bits).  These
+//           scores are approximate and only choose keys: the scores of the eight chosen keys of a row are then
+//           recomputed from the 16-bit inputs.  The threshold of any subset of a row's scores is a lower bound of the
+//           row's threshold (f only grows when entries are added), so a few Newton steps from the left on those eight
+//           values give a lower bound `lo` that lies within a few hundredths (in z) of the threshold for such rows,
+//           whichever keys were chosen.
 //   walk 2  the same products with the accumulators preloaded with -lo; a lane whose eight scores of a 16-key half
 //           block have a positive maximum writes those eight values and the half block's index to its event list in
 //           global memory (a per-workgroup slot of the workspace; the events are a few per cent of the scores).
@@ -23,6 +27,8 @@
 // counters in the same XCD-aware order as the dense kernel, longest causal row blocks first, and help the other
 // XCDs when their own counter runs out.
 #pragma once
+#include <type_traits>
+
 #include "attn_kernel.h"
 
 namespace adsp {
@@ -30,11 +36,8 @@ namespace adsp {
 #ifndef ADSP_GATHER_DEPTH
 #define ADSP_GATHER_DEPTH 8
 #endif
-#ifndef ADSP_SPARSE_STAGES
-#define ADSP_SPARSE_STAGES 2
-#endif
 #ifndef ADSP_SPARSE_WAVES
-#define ADSP_SPARSE_WAVES (ADSP_SPARSE_STAGES == 2 ? 4 : 3)
+#define ADSP_SPARSE_WAVES 4
 #endif
 constexpr int kSparseStreamCap = 1616;  // candidates per wave the workspace slot holds (SparseGeo::kListCap is at most this)
 constexpr int kSparseMaxKeys = 65536;   // the lists hold 16-bit key indices
@@ -59,6 +62,14 @@ template <> __device__ __forceinline__ void dot2_chunk<f16_t>(float (&acc)[8], u
 }
 #undef ADSP_DOT2_CHUNK
 
+// two 16-byte chunks of e4m3 values as one operand of the fp8 MFMA (64 values of k per lane pair)
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ f32x16 mfma_fp8(u32x4 a_lo, u32x4 a_hi, const uint32_t* b, f32x16 c) {
+  const i32x8 a = {(int)a_lo[0], (int)a_lo[1], (int)a_lo[2], (int)a_lo[3], (int)a_hi[0], (int)a_hi[1], (int)a_hi[2], (int)a_hi[3]};
+  const i32x8 bb = {(int)b[0], (int)b[1], (int)b[2], (int)b[3], (int)b[4], (int)b[5], (int)b[6], (int)b[7]};
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, bb, c, 0, 0, 0, 0, 0, 0);  // both operands e4m3, no block scales
+}
+
 // inclusive prefix sum over the wave on the DPP network; all 64 lanes active
 __device__ __forceinline__ int wave_scan_i(int v) {
   v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
@@ -76,10 +87,15 @@ template <typename T, int D> struct SparseGeo {
   static constexpr int kBM = 32 * kNW;
   static constexpr int kThreads = 64 * kNW;
   // K stages during the walks, with the waves' event rings behind them; afterwards the whole array holds the
-  // candidate lists.  Two stages: 39 KB, four workgroups per CU (one wave of each per SIMD); three stages (a tile
-  // load has two tile times to arrive): 52 KB at head dim 128, three workgroups per CU.
-  static constexpr int kStages = ADSP_SPARSE_STAGES;
-  static constexpr int kMinLds = kStages == 2 ? 39 * 1024 : 52 * 1024;  // (1 KB left for the small arrays)
+  // candidate lists.  Two stages of 16-bit tiles: 39 KB, four workgroups per CU (one wave of each per SIMD); three
+  // stages (52 KB at head dim 128, three workgroups per CU) measured slower.  The fp8 tiles of the first walk are
+  // half as large and go through the same bytes in four stages.
+  static constexpr int kStages = 2;
+  static constexpr int kStages8 = 4;
+  static constexpr int kK8Row = D;              // bytes per key row of the fp8 tile
+  static constexpr int kK8Tile = kBN * kK8Row;
+  static constexpr int kK8Loads = kK8Tile / 1024;
+  static constexpr int kMinLds = 39 * 1024;  // (1 KB left for the small arrays)
   static constexpr int kLds = kStages * G::kKTile + 4608 > kMinLds ? kStages * G::kKTile + 4608 : kMinLds;  // rings of >= 32 events
   static constexpr int kWaveLds = kLds / kNW;
   // candidates per wave: scores (fp32) and keys (16 bits: the path serves up to 65536 keys) in two arrays, then the
@@ -96,7 +112,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   using G = TileGeo<T, D>;
   using SG = SparseGeo<T, D>;
   using KS = Swz<G::kKRow>;
+  using KS8 = Swz<SG::kK8Row>;
   static_assert(G::k16, "16-bit element types only");
+  static_assert(D % 64 == 0, "the fp8 products take 64 values of the head dim at a time");
   static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
   constexpr int NW = SG::kNW, BM = SG::kBM;
   __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
@@ -114,6 +132,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   const long long per_xcd = (total + 7) / 8;
   const float qs = p.qscale, inv_qs = 1.f / p.qscale;
   constexpr int kKPer = (G::kKLoads + NW - 1) / NW;
+  constexpr int kK8Per = SG::kK8Loads / NW;
+  static_assert(SG::kK8Loads % NW == 0 && (NW * 64 / KS8::kC) % 16 == 0, "every wave loads whole KBs of the fp8 tile, with one swizzle");
+  static_assert(SG::kStages8 * SG::kK8Tile <= SG::kStages * G::kKTile, "the fp8 stages lie inside the 16-bit ones");
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
   static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
 
@@ -137,6 +158,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // tile DMA and fragment-read geometry (see attn_fwd_kernel)
     const uint32_t koff = (uint32_t)((wave * 64 + lane) / KS::kC * G::kKRow + ((((wave * 64 + lane) % KS::kC) ^ KS::sw((wave * 64 + lane) / KS::kC)) << 4));
     const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
+    // the same for the fp8 tile: rows of D bytes, a lane's 32 values of a 64-value slice are two adjacent chunks
+    const uint32_t koff8 = (uint32_t)((wave * 64 + lane) / KS8::kC * SG::kK8Row + ((((wave * 64 + lane) % KS8::kC) ^ KS8::sw((wave * 64 + lane) / KS8::kC)) << 4));
+    const uint32_t k8_lane = (uint32_t)(lq * SG::kK8Row + (((2 * lh) ^ KS8::sw(lq)) << 4));
 
     __syncthreads();  // the previous row block is done with LDS and with s_item
     if (tid == 0) {
@@ -225,19 +249,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     const int wave_row0 = m0 + wave * 32;
     const bool live = qi < L;
 
-    // ---- Q fragments; rows past the valid length are zero (their scores are never used) ----------------------
-    uint32_t qf[G::kQRegs];
-    {
-      const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
+    // ---- Q fragments of the first walk, rounded to e4m3: per 64-value slice of the head dim the lane holds the 32
+    // values [32 lh, 32 lh + 32) of its row, in the order of the copy of K.  Rows past the valid length are zero
+    // (their scores are never used). ------------------------------------------------------------------------------
+    const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
+    uint32_t q8[D / 64 * 8];
+    uint32_t qf[G::kQRegs];  // those of the 16-bit products: loaded behind the first walk
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
+    for (int c = 0; c < D / 64; ++c) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = live ? raw[e] : 0u;
+      for (int hq = 0; hq < 4; ++hq) {
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + c * 64 + lh * 32 + hq * 8);
+#pragma unroll
+        for (int e = 0; e < 4; e += 2) {
+          uint32_t w = cvt_e4m3_pair(unpack_lo<T>(raw[e]), unpack_hi<T>(raw[e]), 0u, false);
+          w = cvt_e4m3_pair(unpack_lo<T>(raw[e + 1]), unpack_hi<T>(raw[e + 1]), w, true);
+          q8[c * 8 + hq * 2 + (e >> 1)] = live ? w : 0u;
+        }
       }
     }
 
     const unsigned char* kglob = reinterpret_cast<const unsigned char*>(p.k) + kv_base * 2;
+    const unsigned char* k8glob = p.k8 + (size_t)(b * p.Hkv + kvh) * (size_t)p.Npad * SG::kK8Row;
+    // (the copy is padded to whole tiles, so no tile sticks out)
+    auto issue_k8 = [&](unsigned char* lds, int kt) {
+      const unsigned char* base = uniform_ptr(k8glob + (size_t)kt * SG::kK8Tile);
+#pragma unroll
+      for (int j0 = 0; j0 < kK8Per; ++j0) dma16s(base + j0 * (NW * 1024), koff8, lds + (j0 * NW + wave) * 1024);
+    };
     auto issue_k = [&](unsigned char* lds, int kt) {
       const unsigned char* base = uniform_ptr(kglob + (size_t)kt * G::kKTile);
       if ((kt + 1) * kBN <= N) {
@@ -258,30 +297,63 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // body(kt, tile) over all key tiles of the row block; stops when a lane gave up.  The K tiles go through a ring of
     // kStages LDS buffers: the load of tile t + kStages - 1 is issued behind the barrier that opens tile t (every wave
     // is done with tile t - 1, whose buffer it takes) and has kStages - 1 tile times to arrive.
-    auto walk = [&](auto&& body) {
-      constexpr int kStages = SG::kStages;
+    // (stages_c, tile_c, per_c: the ring's depth, the bytes of a tile and the loads per wave and tile, as constants)
+    auto walk = [&](auto stages_c, auto tile_c, auto per_c, auto&& issue, auto&& body) {
+      constexpr int kStages = decltype(stages_c)::value, kTile = decltype(tile_c)::value, kPer = decltype(per_c)::value;
       __syncthreads();
 #pragma unroll
       for (int s = 0; s < kStages - 1; ++s)
-        if (s < nt) issue_k(lds_all + s * G::kKTile, s);
+        if (s < nt) issue(lds_all + s * kTile, s);
       int stage = 0;  // buffer of tile cur
       for (int cur = 0; cur < nt; ++cur) {
         // this wave's share of tile cur has landed: everything but the loads issued after it (those of the tiles in
         // between; stores issued after it only make the wait longer than needed)
         if (cur + kStages - 1 <= nt) {
           if constexpr (kStages == 2) __builtin_amdgcn_s_waitcnt(0x0f70);
-          else __builtin_amdgcn_s_waitcnt(0x0f70 | ((kStages - 2) * kKPer));
+          else __builtin_amdgcn_s_waitcnt(0x0f70 | ((kStages - 2) * kPer));
         } else {
           __builtin_amdgcn_s_waitcnt(0x0f70);  // the last tiles: nothing was issued behind them
         }
         __syncthreads();
         if (s_giveup[(cur + 1) & 1]) break;  // set while the previous tile was worked on
         const int pre = cur + kStages - 1;
-        if (pre < nt) issue_k(lds_all + (stage == 0 ? kStages - 1 : stage - 1) * G::kKTile, pre);
+        if (pre < nt) issue(lds_all + (stage == 0 ? kStages - 1 : stage - 1) * kTile, pre);
         __builtin_amdgcn_sched_barrier(0);
-        body(cur, lds_all + stage * G::kKTile);
+        body(cur, lds_all + stage * kTile);
         stage = stage + 1 == kStages ? 0 : stage + 1;
       }
+    };
+    // approximate S^T of one tile from the fp8 operands; f(s0, s1) unless no row of the wave sees the tile.  Scores past
+    // a row's last valid key are hugely negative (finite: a position is still to be written into their low bits).
+    auto for_tile8 = [&](int kt, const unsigned char* kt_lds, auto&& f) {
+      if (p.causal && kt * kBN > wave_row0 + 31) return;
+      const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
+      f32x16 s0, s1;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s0[i] = 0.f;
+        s1[i] = 0.f;
+      }
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k8_lane;
+      asm volatile("" : "+v"(ka));
+      u32x4 a0[D / 32], a1[D / 32];
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c) a0[c] = lds_read16(ka ^ (((c >> 1) * 4 + (c & 1)) << 4));
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c) a1[c] = lds_read16(ka ^ (((c >> 1) * 4 + (c & 1)) << 4), 32 * SG::kK8Row);
+#pragma unroll
+      for (int c = 0; c < D / 64; ++c) s0 = mfma_fp8(a0[2 * c], a0[2 * c + 1], q8 + c * 8, s0);
+#pragma unroll
+      for (int c = 0; c < D / 64; ++c) s1 = mfma_fp8(a1[2 * c], a1[2 * c + 1], q8 + c * 8, s1);
+      if (need_mask) {
+        const int jb = kt * kBN + 4 * lh;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s0[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? s0[i] : -1e30f;
+          s1[i] = (jb + 32 + 8 * (i >> 2) + (i & 3) <= lim) ? s1[i] : -1e30f;
+        }
+      }
+      f(s0, s1);
     };
     // S^T of one tile (two 32-key blocks), accumulators preloaded with `init`; f(s0, s1) unless no row of the wave
     // sees the tile.  Scores past a row's last valid key are -inf.
@@ -311,6 +383,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
         s1 = mfma_16bit<T>(a1[ks], bq, s1);
       }
+      // the order of issue: four fragment reads ahead of the first product, then one read behind every product
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * (D / 16) - 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
       if (need_mask) {
         const int jb = kt * kBN + 4 * lh;
 #pragma unroll
@@ -336,14 +416,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // z) of the lane's running maximum, the row block is given up before the walk is over.  A heuristic that only
     // decides which kernel does the work.
     int near_cnt = 0;
-    walk([&](int kt, const unsigned char* kt_lds) {
-      for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
-        float m0v = s0[0], m1v = s1[0];
+    // A score carries its position in the low 15 bits of its mantissa (4: which of the lane's 16 values of the block,
+    // 11: the 32-key block), so the maxima know their keys at the price of one instruction per score; the approximate
+    // scores have fewer than nine good mantissa bits anyway.
+    auto tagged = [](float x, uint32_t bits, uint32_t tag) { return __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, x) & ~bits) | tag); };
+    walk(std::integral_constant<int, SG::kStages8>{}, std::integral_constant<int, SG::kK8Tile>{}, std::integral_constant<int, kK8Per>{}, issue_k8, [&](int kt, const unsigned char* kt_lds) {
+      for_tile8(kt, kt_lds, [&](const f32x16& s0, const f32x16& s1) {
+        float m0v = tagged(s0[0], 15u, 0u), m1v = tagged(s1[0], 15u, 0u);
 #pragma unroll
         for (int i = 1; i < 16; ++i) {
-          m0v = fmaxf(m0v, s0[i]);
-          m1v = fmaxf(m1v, s1[i]);
+          m0v = fmaxf(m0v, tagged(s0[i], 15u, (uint32_t)i));
+          m1v = fmaxf(m1v, tagged(s1[i], 15u, (uint32_t)i));
         }
+        m0v = tagged(m0v, 0x7ff0u, (uint32_t)(2 * kt) << 4);
+        m1v = tagged(m1v, 0x7ff0u, (uint32_t)(2 * kt + 1) << 4);
         keep_top(m0v);
         keep_top(m1v);
         if (kt >= 6 && kt < 12) {
@@ -367,9 +453,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // ---- lower bound of the row's threshold from its eight kept values (raw score units) --------------------
     // f(t) = qs^2 sum (r - t)_+^2 - 1 (alpha 1.5) or qs sum (r - t)_+ - 1 (alpha 2) is convex and decreasing and
     // f(max - 1 / qs) >= 0, so Newton from there approaches the subset's root from the left and never passes it.
+    // ---- Q fragments of the 16-bit products ----------------------------------------------------------------------
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = live ? raw[e] : 0u;
+    }
+    // ---- the scores of the row's eight chosen keys from the 16-bit inputs, with the products of the second walk: in
+    // product m the A operand's row i is the key that row i chose as its m-th (a lane fetches its slice of that key's
+    // row from memory), so the diagonal of S^T holds the wanted scores, bit for bit those the second walk will see
+    // ----------------------------------------------------------------------------------------------------------------
+    float r[8];
+    {
+      const uint32_t u[4] = {__builtin_bit_cast(uint32_t, t1), __builtin_bit_cast(uint32_t, t2), __builtin_bit_cast(uint32_t, t3), __builtin_bit_cast(uint32_t, t4)};
+      uint32_t pu[4];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) pu[m] = (uint32_t)__shfl_xor((int)u[m], 32, 64);
+      const int diag = ((lq >> 3) << 2) | (lq & 3);  // which of the lane's 16 values of a block belongs to key lq of the block,
+      const bool diag_here = lh == ((lq >> 2) & 1);  // and which of the row's two lanes holds it
+      constexpr int kBatch = D / 16;
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        // the row's first lane chose keys 0 .. 3, its second lane keys 4 .. 7
+        const uint32_t w = ((m < 4) == (lh == 0)) ? u[m & 3] : pu[m & 3];
+        const bool ok = __builtin_bit_cast(float, w) > -1e29f;  // fewer than four valid keys leave -inf or masked entries behind
+        uint32_t key = ((w >> 4) & 0x7ffu) * 32u + 8u * ((w & 15u) >> 2) + (w & 3u) + (m < 4 ? 0u : 4u);
+        key = (ok && key < (uint32_t)N) ? key : 0u;
+        const unsigned char* krow = kglob + (size_t)key * G::kKRow + 16 * lh;
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int k0 = 0; k0 < D / 16; k0 += kBatch) {
+          u32x4 kv[kBatch];
+#pragma unroll
+          for (int j = 0; j < kBatch; ++j) kv[j] = *reinterpret_cast<const u32x4*>(krow + (k0 + j) * 32);
+#pragma unroll
+          for (int j = 0; j < kBatch; ++j) {
+            const int ks = k0 + j;
+            acc = mfma_16bit<T>(kv[j], u32x4{qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]}, acc);
+          }
+        }
+        // (the order of issue: a key's loads together, then its products)
+        __builtin_amdgcn_sched_group_barrier(0x020, D / 16, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, D / 16, 0);
+        float d = acc[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) d = diag == i ? acc[i] : d;
+        const float other = __shfl_xor(d, 32, 64);
+        d = diag_here ? d : other;
+        r[m] = ok ? d : -INFINITY;
+      }
+    }
     float lo_raw;
     {
-      float r[8] = {t1, t2, t3, t4, __shfl_xor(t1, 32, 64), __shfl_xor(t2, 32, 64), __shfl_xor(t3, 32, 64), __shfl_xor(t4, 32, 64)};
       const float rmax = fmaxf(r[0], r[4]);
       float t = rmax - inv_qs;
       const float target = (AM == ATT_15) ? inv_qs * inv_qs : inv_qs;
@@ -466,7 +604,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
     };
-    walk([&](int kt, const unsigned char* kt_lds) {
+    walk(std::integral_constant<int, SG::kStages>{}, std::integral_constant<int, G::kKTile>{}, std::integral_constant<int, kKPer>{}, issue_k, [&](int kt, const unsigned char* kt_lds) {
       for_tile(kt, kt_lds, -lo_raw, [&](const f32x16& s0, const f32x16& s1) {
         float h00 = s0[0], h01 = s0[8], h10 = s1[0], h11 = s1[8];
 #pragma unroll

@@ -40,6 +40,13 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   f32x2 f = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
 }
+// two floats -> two e4m3 bytes in the low (hi = false) or high half of `old`; saturating at the format's largest value
+__device__ __forceinline__ uint32_t cvt_e4m3_pair(float a, float b, uint32_t old, bool hi) {
+  a = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
+  b = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
+  return hi ? (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true) : (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, false);
+}
+
 template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
 template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
 template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w << 16); }

@@ -166,9 +166,10 @@ def test_sizing_helpers_and_status_strings():
     # ... and at head dims 64 / 128 the sparse-support kernel's counters, flags and candidate slots (at most 1024)
     vt = 8 * 8 * 128 * 8192 * 2
     slot = 4 * 1616 * 8
-    assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) == vt + 256 + 768 + 8 * 32 * 64 * 4 + 1024 * slot  # (8 * 8 + 1) hint pairs, padded to 256
+    k8 = 8 * 8 * 8192 * 128  # the one-byte copy of K
+    assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) == vt + 256 + 768 + 8 * 32 * 64 * 4 + 1024 * slot + k8  # (8 * 8 + 1) hint pairs, padded to 256
     small = lib.adsp_attn_workspace_bytes(1, 2, 2, 128, 64, _lib.ADSP_F16)
-    assert 8 * slot < small < 8 * slot + 2 * 64 * 128 * 2 + 1024
+    assert 8 * slot < small < 8 * slot + 2 * 64 * 128 * 3 + 1024
     assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_F32) == 0
     assert lib.adsp_attn_bmask_words(8192) == 64 * 4 and lib.adsp_attn_bmask_words(64) == 1
     assert lib.adsp_status_string(0) == b"ok"
