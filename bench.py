@@ -35,16 +35,17 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these
 # same workloads, each counter scaled by what it reads for a plain 1 GiB copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
-MEASURED_HBM_TRAFFIC_BYTES = {"c4": 1.511e9, "c3": 0.1998e9, "c5": 0.632e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5373e9,
-                              "c2_bwd_f32": 1.0848e9, "c2_bwd_bf16": 0.5476e9,
-                              "c4_bwd": 23.57e9}  # c4_bwd: dq kernel 2.03e9 + dk/dv kernel 21.54e9
+MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.508e9, "c3": 0.1802e9, "c5": 0.620e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5371e9,
+                              "c2_bwd_f32": 1.0847e9, "c2_bwd_bf16": 0.5476e9,
+                              "c4_bwd": 22.59e9}  # c4_bwd: dq kernel 2.02e9 + dk/dv kernel 20.58e9
 
 
-# The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
-# probe of the score distribution, the sparse-support kernel, the key-major copy of V and the dense kernel, of which
-# the last two return at once unless the sparse-support kernel left row blocks over (c3: the probe marks every head
-# dense and the dense kernel does all the work).
-FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + this + V copy and attn_fwd_kernel on leftovers)",
+# The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is five launches: a
+# probe of the score distribution, the one-byte copy of K, the sparse-support kernel, the key-major copy of V and the
+# dense kernel, of which the last two return at once unless the sparse-support kernel left row blocks over (c3: the
+# probe marks every head dense, the copy of K and the sparse-support kernel step aside and the dense kernel does all
+# the work).
+FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + fp8 copy of K + this + V copy and attn_fwd_kernel on leftovers)",
                "c3": "attn_fwd_kernel<bf16, 64, single step> (step = probe + sparse-support kernel stepping aside + V copy + this)",
                "c5": "attn_fwd_kernel<bf16, 64, generic alpha, candidate lists>"}
 
