@@ -63,32 +63,32 @@ __device__ __forceinline__ float hist_surrogate(const float (&cnt)[BINS], float 
   return acc - 1.f;
 }
 
-// Starting point inside [a, c]: root (nearest c) of the parabola through the surrogate at a, mid, c
-// (triton_entmax_v2.py:208-322).
+// Starting point inside [a, c]: one step of Muller's method on the surrogate, through a, the midpoint and c (the
+// reference starts from the same parabola, triton_entmax_v2.py:208-322).  Written around c with divided differences:
+// p(x) = fc + w (x - c) + q (x - c)^2, root x = c - 2 fc / (w +- sqrt(w^2 - 4 fc q)) with the sign that makes the
+// denominator larger, i.e. the root nearer to c, which also covers a vanishing curvature (x = c - fc / w).  Without a
+// real root: the secant through the two ends; the midpoint when that fails too.  The result is clamped to [a, c]; it
+// only seeds the iteration.
 template <int BINS>
 __device__ __forceinline__ float hist_start_point(const float (&cnt)[BINS], float t_shift, float a, float c) {
-  const float EPS = 1e-10f;
-  float b = 0.5f * (a + c);
-  float fa = hist_surrogate<BINS>(cnt, t_shift, a);
-  float fb = hist_surrogate<BINS>(cnt, t_shift, b);
-  float fc = hist_surrogate<BINS>(cnt, t_shift, c);
-  float den = (a - b) * (a - c) * (b - c);
-  float A = (fa * (b - c) + fb * (c - a) + fc * (a - b)) / den;
-  float B = (fa * (c * c - b * b) + fb * (a * a - c * c) + fc * (b * b - a * a)) / den;
-  float C = (fa * b * c * (b - c) + fb * a * c * (c - a) + fc * a * b * (a - b)) / den;
-  float mid = 0.5f * (a + c);
-  float x_lin = fabsf(B) > EPS ? -C / B : mid;
-  float disc = B * B - 4.f * A * C;
-  float sq = sqrtf(fmaxf(disc, 0.f));
-  float r1 = (-B + sq) / (2.f * A), r2 = (-B - sq) / (2.f * A);
-  bool v1 = r1 >= a && r1 <= c, v2 = r2 >= a && r2 <= c;
-  float x_quad = (v1 && v2) ? (fabsf(c - r1) <= fabsf(c - r2) ? r1 : r2) : (v1 ? r1 : (v2 ? r2 : mid));
-  float sden = fc - fa;
-  float x_sec = fabsf(sden) > EPS ? c - fc * (c - a) / sden : mid;
-  x_quad = disc >= 0.f ? x_quad : x_sec;
-  float x = fabsf(A) < EPS ? x_lin : x_quad;
-  x = fabsf(den) < EPS ? mid : x;
-  x = (x == x) ? x : mid;  // NaN guard
+  const float b = 0.5f * (a + c), h = c - b;
+  if (!(h > 0.f)) return b;
+  const float fa = hist_surrogate<BINS>(cnt, t_shift, a);
+  const float fb = hist_surrogate<BINS>(cnt, t_shift, b);
+  const float fc = hist_surrogate<BINS>(cnt, t_shift, c);
+  const float d1 = (fb - fa) / h, d2 = (fc - fb) / h;  // slopes of the two halves
+  const float q = (d2 - d1) / (2.f * h);               // half the curvature
+  const float w = d2 + q * h;                          // slope of the parabola at c
+  const float disc = w * w - 4.f * fc * q;
+  float x = b;
+  if (disc >= 0.f) {
+    const float root = sqrtf(disc);
+    const float den = w >= 0.f ? w + root : w - root;
+    if (den != 0.f) x = c - 2.f * fc / den;
+  } else if (fc != fa) {
+    x = c - fc * (c - a) / (fc - fa);
+  }
+  x = (x == x) ? x : b;  // (0 / 0 and inf - inf end here)
   return fminf(fmaxf(x, a), c);
 }
 
