@@ -81,9 +81,10 @@ int adsp_entmax_rows_bwd(const void* y, const void* dy, void* dx, int64_t rows, 
 
 /*
  * Bytes of scratch the forward entry points need for these dimensions; 0 for fp32.  For the 16-bit types: a
- * key-major copy of V and, at head dims 64 and 128, the work counters, row-block flags and event slots of the
- * sparse-support kernel (up to 1024 slots of 51 KiB; sequences of up to 65536 keys).  The buffer must be 16-byte aligned device memory; its
- * contents need not survive between calls.  For the block-mask variant pass Hq = Hkv = H.
+ * key-major copy of V and, at head dims 64 and 128, the work counters, row-block flags and candidate streams of the
+ * sparse-support kernel (up to 1024 slots of 51 KiB; sequences of up to 65536 keys) and a one-byte (fp8 e4m3) copy
+ * of K.  The buffer must be 16-byte aligned device memory; its contents need not survive between calls, and two
+ * calls that run at the same time need a buffer each.  For the block-mask variant pass Hq = Hkv = H.
  */
 size_t adsp_attn_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
 
@@ -98,7 +99,9 @@ size_t adsp_attn_bmask_words(int N);
  *            bit (c % 32) of word c / 32 of a row block = key tile c holds a non-zero probability.
  *   varlen : NULL, or [B] valid lengths as int32 (varlen_bits = 32) or int64 (varlen_bits = 64);
  *            keys >= length are masked, output rows >= length are written as zeros.
- *   niter  : Halley/bisection refinement passes after the histogram bracket (>= 0).
+ *   niter  : Halley/bisection refinement passes after the histogram bracket (>= 0).  fp32 takes niter + 1 of them,
+ *            as the reference does (adasplash/adasplash_v2.py:567-611 and :617-681); the 16-bit types take niter on
+ *            the dense kernel, and the sparse-support kernel (head dims 64 / 128) iterates to convergence.
  * Replaces the four launches at adasplash/adasplash_v2.py:1288-1419.
  */
 int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
@@ -108,7 +111,7 @@ int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, void* out, flo
 /*
  * adsp_attn_v2_fwd without a workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
- * scratch memory (key-major copy of V, control words, flags and candidate streams of the sparse-support kernel)
+ * scratch memory (key-major copy of V, control words, flags, candidate streams and fp8 copy of K of the sparse-support kernel)
  * lives in a device array inside the library, 64 MiB on every GPU the library runs on, held until the process ends;
  * problems whose adsp_attn_workspace_bytes() exceeds adsp_attn_v2_fwd_noalloc_max_bytes() are rejected with
  * ADSP_ERR_TOO_LARGE.  The call allocates and frees nothing and records no memset (the kernels clear what must start
