@@ -113,6 +113,29 @@ def test_heads_of_one_batch_can_go_different_ways(sparse_switch):
     assert max_err(forward(q, k, v)[0], want) < 2e-2
 
 
+@pytest.mark.parametrize("dtype,qscale,kscale", [
+    (torch.bfloat16, 600.0, 1.0),     # q beyond the one-byte format's largest value: saturated in the first walk
+    (torch.bfloat16, 1.0, 1000.0),    # the same for the copy of K
+    (torch.bfloat16, 30.0, 1.0 / 512),  # k below the format's smallest value: the copy of K is all zeros
+    (torch.float16, 1.0 / 300, 40.0),   # q vanishes in one byte, k does not
+    (torch.float16, 16.0, 16.0),        # large but representable
+])
+def test_badly_scaled_inputs_only_cost_speed(sparse_switch, dtype, qscale, kscale):
+    """The first walk reads q and k rounded to one byte (e4m3: largest value 448, smallest 2^-9) and only chooses
+    keys; whatever it chooses, the bound it leads to is valid, so inputs far outside that range must still give the
+    oracle's answer (through more candidates or through the dense kernel).  The products q k stay of order one or
+    larger here, so the supports are short."""
+    q, k, v = qkv(1, 2, 1, 1024, 128, dtype, seed=21)
+    q = (q.float() * qscale).to(dtype)
+    k = (k.float() * kscale).to(dtype)
+    varlen = torch.tensor([1000], dtype=torch.int32)
+    want = exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)
+    sparse_switch(True)
+    out = forward(q, k, v, varlen)[0]
+    assert torch.isfinite(out.float()).all()
+    assert max_err(out, want) < 2e-2
+
+
 @pytest.mark.parametrize("alpha,causal", [(1.5, False), (2.0, False), (2.0, True)])
 def test_block_mask_entry_point_takes_the_same_path(sparse_switch, alpha, causal):
     q, k, v = qkv(2, 2, 2, 640, 64, torch.bfloat16, seed=7, scale=2.0)
