@@ -55,6 +55,7 @@ def units():
             out.append((f"attn_bwd_{tag}_d{d}", "attn_bwd_unit.hip", base))
             if tag != "f32" and d in (64, 128):
                 out.append((f"attn_sparse_{tag}_d{d}", "attn_sparse_unit.hip", base + ATTN_FLAGS))
+                out.append((f"attn_bwd_sparse_{tag}_d{d}", "attn_bwd_sparse_unit.hip", base + ATTN_FLAGS))
     return out
 
 

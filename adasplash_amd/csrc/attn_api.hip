@@ -23,6 +23,11 @@ int launch_attn_sparse_bf16_d64(const AttnParams&, int, int, hipStream_t);
 int launch_attn_sparse_bf16_d128(const AttnParams&, int, int, hipStream_t);
 int launch_attn_sparse_f16_d64(const AttnParams&, int, int, hipStream_t);
 int launch_attn_sparse_f16_d128(const AttnParams&, int, int, hipStream_t);
+// attn_bwd_dq_sparse_kernel (attn_bwd_sparse_unit.hip): likewise
+int launch_attn_bwd_sparse_bf16_d64(const AttnBwdParams&, int, int, hipStream_t);
+int launch_attn_bwd_sparse_bf16_d128(const AttnBwdParams&, int, int, hipStream_t);
+int launch_attn_bwd_sparse_f16_d64(const AttnBwdParams&, int, int, hipStream_t);
+int launch_attn_bwd_sparse_f16_d128(const AttnBwdParams&, int, int, hipStream_t);
 
 typedef int (*attn_fwd_fn)(const AttnParams&, int, hipStream_t);
 typedef int (*attn_bwd_fn)(const AttnBwdParams&, int, hipStream_t);
@@ -398,9 +403,36 @@ extern "C" int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, voi
                            0, workspace, workspace_bytes, tile_counts, (hipStream_t)stream);
 }
 
+namespace adsp {
+// Workspace of the backward for the 16-bit types: the tile-wise transposed copies of k, q and dout, then -- for the
+// head dims the sparse-support dQ kernel serves -- its work counters, per-row-block flags and candidate streams (the
+// forward's layout without the copy of K).
+struct BwdWorkspace {
+  size_t copies_bytes, queue_off, flags_off, events_off, total;
+  int slots;  // 0: no sparse-support kernel for these dimensions
+};
+static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
+  BwdWorkspace w = {};
+  if (dtype == ADSP_F32) return w;
+  w.copies_bytes = (size_t)B * (Hkv + 2 * (size_t)Hq) * D * npad_of(N) * 2;
+  w.total = w.copies_bytes;
+  if ((D == 64 || D == 128) && N <= 65536) {
+    const long long items = (long long)B * Hq * mblocks_of(N);
+    long long slots = (items + 7) / 8 * 8;
+    if (slots > kSparseMaxSlots) slots = kSparseMaxSlots;
+    w.slots = (int)slots;
+    w.queue_off = align256(w.copies_bytes);
+    w.flags_off = align256(w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8);
+    w.events_off = align256(w.flags_off + (size_t)items * 4);
+    w.total = w.events_off + (size_t)slots * kSparseSlotBytes;
+  }
+  return w;
+}
+}  // namespace adsp
+
 extern "C" size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype) {
   if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
-  return (size_t)B * (Hkv + 2 * (size_t)Hq) * D * adsp::npad_of(N) * 2;
+  return adsp::bwd_workspace(B, Hq, Hkv, N, D, dtype).total;
 }
 
 extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* taus,
@@ -445,11 +477,16 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   p.qscale = (float)((alpha - 1.0) / sqrt((double)D));
   p.sm_scale = (float)(1.0 / sqrt((double)D));
   p.c0 = (float)(1.0 / (alpha - 1.0));
+  p.block_flags = nullptr;
+  p.queue = nullptr;
+  p.hints = nullptr;
+  p.events = nullptr;
   const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
 
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
-    const size_t need = adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dtype);
+    const BwdWorkspace w = bwd_workspace(B, Hq, Hkv, N, D, dtype);
+    const size_t need = w.total;
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
     uint16_t* kt = (uint16_t*)workspace;
     uint16_t* qt = kt + (size_t)B * Hkv * D * p.Npad;
@@ -464,6 +501,38 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     p.kt = kt;
     p.qt = qt;
     p.dot = dot;
+    // Sparse-support dQ kernel first (alpha 1.5 / 2): it serves the row blocks whose supports are short and flags the
+    // others for attn_bwd_dq_kernel below; the dK/dV kernel reads delta and 1 / sum p from whichever of the two wrote them.
+    const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
+    if (sparse) {
+      unsigned char* ws = (unsigned char*)workspace;
+      p.queue = (uint32_t*)(ws + w.queue_off);
+      p.hints = p.queue + 64;
+      p.block_flags = (int32_t*)(ws + w.flags_off);
+      p.events = ws + w.events_off;
+      AttnParams pp = {};  // what the probe reads: q, k, lengths, dimensions, scale and the control words it clears
+      pp.q = q;
+      pp.k = k;
+      pp.varlen = varlen;
+      pp.varlen_bits = varlen_bits;
+      pp.B = B;
+      pp.Hq = Hq;
+      pp.Hkv = Hkv;
+      pp.N = N;
+      pp.causal = p.causal;
+      pp.qscale = p.qscale;
+      pp.queue = p.queue;
+      pp.hints = p.hints;
+      int rc;
+      if (dtype == ADSP_BF16) {
+        hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, pp, D, am);
+        rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, w.slots, s);
+      } else {
+        hipLaunchKernelGGL(attn_probe_kernel<f16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, pp, D, am);
+        rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, w.slots, s);
+      }
+      if (rc != 0) return ADSP_ERR_LAUNCH;
+    }
   }
   int rc = kBwdTable[dtype][head_dim_slot(D)](p, am, s);
   if (rc != 0) return ADSP_ERR_LAUNCH;

@@ -312,6 +312,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int h = kvh * group + in_unit % group;
   const int bh = b * p.Hq + h;
+  // behind the sparse-support dQ kernel: only the row blocks it flagged (all of them when it stepped aside)
+  if (p.block_flags && p.queue[kCtrlAllDense] == 0u && (p.queue[kCtrlFlagged] == 0u || p.block_flags[(size_t)bh * n_blk + mblk] == 0)) return;
   const int L = bwd_seq_len(p, b);
   const int m0 = mblk * kBwdRows;
   const int wave_row0 = m0 + wave * 32;

@@ -20,6 +20,11 @@ struct AttnBwdParams {
   float qscale;    // (alpha - 1) / sqrt(D)
   float sm_scale;  // 1 / sqrt(D)
   float c0;        // 1 / (alpha - 1)
+  // the sparse-support dQ kernel and its hand-over to the dense one (null: dense kernels only), as in AttnParams
+  int32_t* block_flags;   // [B, Hq, n_mblk] 1 = row block left to attn_bwd_dq_kernel
+  uint32_t* queue;        // control words: work counters, flagged count, "every head dense"
+  uint32_t* hints;        // two counters per K/V head and one pair over all heads
+  unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
 };
 
 }  // namespace adsp

@@ -1,0 +1,533 @@
+// dQ of the sparse entmax attention from the rows' supports (gfx950, 16-bit inputs, alpha = 1.5 / 2, head dims 64 / 128):
+// the backward's counterpart of attn_fwd_sparse_kernel.
+//
+// The forward left every row's threshold tau.  With it the support needs no search: one 16-bit score walk with the
+// accumulators preloaded with -tau collects exactly the keys with a non-zero probability (the forward's second walk,
+// with the threshold itself in place of a lower bound), a counting sort turns the wave's stream into per-row lists, and
+// the rest is row-wise arithmetic on those few keys:
+//   dP_ij = dO_i . v_j,  delta_i = sum_j u_ij dP_ij / sum_j u_ij,  dQ_i = sum_j u_ij (dP_ij - delta_i) k_j / sqrt(D)
+// with u = p^(2 - alpha).  A group of D / 8 lanes serves a row: each lane holds eight columns of dO_i, fetches its
+// 16 bytes of v_j and k_j, the group adds up the partial dot products on the DPP network, and since delta_i is only
+// known at the end the lanes keep two sums, A = sum u dP k and B = sum u k: dQ_i = (A - delta_i B) / sqrt(D).  Weights
+// and sums are fp32.  delta_i and 1 / sum_j p_ij go to the arrays the dK/dV kernel reads.
+//
+// Row blocks whose supports outgrow the stream or the lists are flagged and left to attn_bwd_dq_kernel, launched
+// behind, exactly as in the forward; the kernel is persistent and draws row blocks from the same per-XCD counters.
+#pragma once
+#include "attn_bwd_kernel.h"
+#include "attn_sparse_kernel.h"
+
+namespace adsp {
+
+// sum over a group of LANES (8 or 16) adjacent lanes, left in every lane of the group
+template <int LANES> __device__ __forceinline__ float group_sum(float x) {
+  if constexpr (LANES == 16) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xf, 0xf, false));  // row_mirror
+  }
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  return x;
+}
+
+template <typename T, int D, int AM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE_WAVES, ADSP_SPARSE_WAVES))) void attn_bwd_dq_sparse_kernel(AttnBwdParams p) {
+  using G = TileGeo<T, D>;
+  using SG = SparseGeo<T, D>;
+  using KS = Swz<G::kKRow>;
+  static_assert(G::k16, "16-bit element types only");
+  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  constexpr int NW = SG::kNW, BM = SG::kBM;
+  __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
+  __shared__ int s_item, s_skip;
+  // a lane ran out of event slots, or a wave out of list room.  Two words: the walks write the one of the tile's
+  // parity and read the other one behind the next barrier, so no wave can read a word another one is still setting
+  __shared__ uint32_t s_giveup[2];
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int N = p.N;
+  const int n_mblk = (N + BM - 1) / BM;
+  const int group = p.Hq / p.Hkv;
+  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
+  const long long per_xcd = (total + 7) / 8;
+  const float qs = p.qscale, inv_qs = 1.f / p.qscale;
+  constexpr int kKPer = (G::kKLoads + NW - 1) / NW;
+  constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
+  static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
+
+  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all row blocks
+    const int units = p.B * p.Hkv;
+    int unmarked = 0;
+    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints[2 * u] < (1u << 20) ? 1 : 0;
+    if (__syncthreads_count(unmarked) == 0) {
+      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue[kCtrlAllDense] = 1u;
+      return;
+    }
+  }
+  int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
+  int known_unit = -1;   // thread 0: the K/V head whose hint counters it has last seen (or set) as served
+  for (;;) {
+    // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
+    // of this loop they would stay live through both walks, and the walks have no registers to spare.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+    // tile DMA and fragment-read geometry (see attn_fwd_kernel)
+    const uint32_t koff = (uint32_t)((wave * 64 + lane) / KS::kC * G::kKRow + ((((wave * 64 + lane) % KS::kC) ^ KS::sw((wave * 64 + lane) / KS::kC)) << 4));
+    const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
+
+    __syncthreads();  // the previous row block is done with LDS and with s_item
+    if (tid == 0) {
+      int got = -1;
+      while (queues_tried < 8) {
+        const int x = ((int)(blockIdx.x & 7) + queues_tried) & 7;
+        const long long i = (long long)atomicAdd(&p.queue[x], 1u);
+        const long long logical = (long long)x * per_xcd + i;
+        if (i < per_xcd && logical < total) {
+          got = (int)logical;
+          break;
+        }
+        ++queues_tried;
+      }
+      s_item = got;
+      s_skip = 0;
+      if (got >= 0) {  // the K/V head of the row block, as decoded below
+        int unit = got / (group * n_mblk);
+        const int units = p.B * p.Hkv;
+        if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
+        if (unit != known_unit) {
+          const uint32_t gave_up = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t served = __hip_atomic_load(p.hints + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
+          const uint32_t all_gave_up = __hip_atomic_load(p.hints + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t all_served = __hip_atomic_load(p.hints + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          s_skip = ((gave_up >= 3u && served == 0u) || (all_gave_up >= 64u && all_served == 0u)) ? 1 : 0;
+          if (served > 0u) known_unit = unit;
+        }
+      }
+      s_giveup[0] = 0u;
+      s_giveup[1] = 0u;
+    }
+    __syncthreads();
+    const int logical = s_item;
+    if (logical < 0) break;
+
+    // ---- row block -> (batch, kv head, row block, head in group), as in attn_fwd_kernel ---------------------
+    const int hg = logical % group;
+    const int mi = (logical / group) % n_mblk;
+    int bkv = logical / (group * n_mblk);
+    {
+      const int units = p.B * p.Hkv;
+      if (units % 8 == 0) bkv = (bkv % (units / 8)) * 8 + bkv / (units / 8);
+    }
+    const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
+    const int h = kvh * group + hg;
+    const int mblk = n_mblk - 1 - mi;
+    const int m0 = mblk * BM;
+    int L = N;
+    if (p.varlen) {
+      long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
+      L = (int)(l < 0 ? 0 : (l > N ? N : l));
+    }
+    int32_t* const flag = p.block_flags + ((size_t)(b * p.Hq + h) * n_mblk + mblk);
+    // Row blocks of one K/V head tend to share their fate: once a few of them were given up and none succeeded, the
+    // rest go to the dense kernel unseen (a hint only: thread 0 read the counters, without any ordering, above).
+    uint32_t* const hint = p.hints + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
+    const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
+    const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
+    const int qi = m0 + wave * 32 + lq;
+
+    if (m0 >= L) {  // row block entirely inside the padding: zero gradient
+      constexpr int kRowDw = D * 2 / 4;
+      uint32_t* o32 = reinterpret_cast<uint32_t*>(p.dq) + (qo_base + (size_t)m0 * D) * 2 / 4;
+      const int rows = (N - m0) < BM ? (N - m0) : BM;
+      for (int i = tid; i < rows * kRowDw; i += SG::kThreads) o32[i] = 0u;
+      if (tid == 0) *flag = 0;
+      continue;
+    }
+
+    if (s_skip) {
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(&p.queue[kCtrlFlagged], 1u);
+      }
+      continue;
+    }
+    const int row_hi = (m0 + BM < L ? m0 + BM : L);
+    const int nt = p.causal ? (row_hi + kBN - 1) / kBN : (L + kBN - 1) / kBN;
+    const int lim = p.causal ? (qi < L - 1 ? qi : L - 1) : L - 1;
+    const int wave_row0 = m0 + wave * 32;
+    const bool live = qi < L;
+
+    // ---- Q fragments; rows past the valid length are zero (their scores are never used).  The forward's threshold
+    // in raw score units: the walk's accumulators start at its negative, so a positive result is a member of the
+    // support ----------------------------------------------------------------------------------------------------
+    const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
+    uint32_t qf[G::kQRegs];
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = live ? raw[e] : 0u;
+    }
+    const float lo_raw = live ? p.taus[(size_t)(b * p.Hq + h) * N + qi] * inv_qs : INFINITY;
+
+    const unsigned char* kglob = reinterpret_cast<const unsigned char*>(p.k) + kv_base * 2;
+    auto issue_k = [&](unsigned char* lds, int kt) {
+      const unsigned char* base = uniform_ptr(kglob + (size_t)kt * G::kKTile);
+      if ((kt + 1) * kBN <= N) {
+#pragma unroll
+        for (int j0 = 0; j0 < kKPer; ++j0) dma16s(base + j0 * (NW * 1024), koff, lds + (j0 * NW + wave) * 1024);
+      } else {  // the last tile sticks out of the tensor: rows past the end are masked later, any valid row will do
+        const unsigned char* g = uniform_ptr(kglob);
+        const int row0 = (int)(koff / G::kKRow);
+        const uint32_t coff = koff % G::kKRow;
+#pragma unroll
+        for (int j0 = 0; j0 < kKPer; ++j0) {
+          int gk = kt * kBN + row0 + j0 * (NW * 64 / KS::kC);
+          gk = gk < N ? gk : N - 1;
+          dma16s(g, (uint32_t)gk * (uint32_t)G::kKRow + coff, lds + (j0 * NW + wave) * 1024);
+        }
+      }
+    };
+    // body(kt, tile) over all key tiles of the row block; stops when a lane gave up.  The K tiles go through a ring of
+    // kStages LDS buffers: the load of tile t + kStages - 1 is issued behind the barrier that opens tile t (every wave
+    // is done with tile t - 1, whose buffer it takes) and has kStages - 1 tile times to arrive.
+    // (stages_c, tile_c, per_c: the ring's depth, the bytes of a tile and the loads per wave and tile, as constants)
+    auto walk = [&](auto stages_c, auto tile_c, auto per_c, auto&& issue, auto&& body) {
+      constexpr int kStages = decltype(stages_c)::value, kTile = decltype(tile_c)::value, kPer = decltype(per_c)::value;
+      __syncthreads();
+#pragma unroll
+      for (int s = 0; s < kStages - 1; ++s)
+        if (s < nt) issue(lds_all + s * kTile, s);
+      int stage = 0;  // buffer of tile cur
+      for (int cur = 0; cur < nt; ++cur) {
+        // this wave's share of tile cur has landed: everything but the loads issued after it (those of the tiles in
+        // between; stores issued after it only make the wait longer than needed)
+        if (cur + kStages - 1 <= nt) {
+          if constexpr (kStages == 2) __builtin_amdgcn_s_waitcnt(0x0f70);
+          else __builtin_amdgcn_s_waitcnt(0x0f70 | ((kStages - 2) * kPer));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);  // the last tiles: nothing was issued behind them
+        }
+        __syncthreads();
+        if (s_giveup[(cur + 1) & 1]) break;  // set while the previous tile was worked on
+        const int pre = cur + kStages - 1;
+        if (pre < nt) issue(lds_all + (stage == 0 ? kStages - 1 : stage - 1) * kTile, pre);
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, lds_all + stage * kTile);
+        stage = stage + 1 == kStages ? 0 : stage + 1;
+      }
+    };
+    // S^T of one tile (two 32-key blocks), accumulators preloaded with `init`; f(s0, s1) unless no row of the wave
+    // sees the tile.  Scores past a row's last valid key are -inf.
+    auto for_tile = [&](int kt, const unsigned char* kt_lds, float init, auto&& f) {
+      if (p.causal && kt * kBN > wave_row0 + 31) return;
+      const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
+      f32x16 s0, s1;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s0[i] = init;
+        s1[i] = init;
+      }
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
+      asm volatile("" : "+v"(ka));
+      u32x4 a0[D / 16], a1[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a0[ks] = lds_read16(ka ^ (ks << 5));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a1[ks] = lds_read16(ka ^ (ks << 5), 32 * G::kKRow);
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s0 = mfma_16bit<T>(a0[ks], bq, s0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s1 = mfma_16bit<T>(a1[ks], bq, s1);
+      }
+      // the order of issue: four fragment reads ahead of the first product, then one read behind every product
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * (D / 16) - 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      if (need_mask) {
+        const int jb = kt * kBN + 4 * lh;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s0[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? s0[i] : -INFINITY;
+          s1[i] = (jb + 32 + 8 * (i >> 2) + (i & 3) <= lim) ? s1[i] : -INFINITY;
+        }
+      }
+      f(s0, s1);
+    };
+
+    // ---- the walk: collect the scores above the threshold ---------------------------------------------------------
+    // A lane whose eight scores of a 16-key half block have a positive maximum puts them, with a tag, into the wave's
+    // ring in LDS (slots are handed out with a ballot: no atomics).  When the ring is full the wave empties it, one
+    // event per lane: the positive entries go to the wave's candidate stream in global memory as (score - threshold, key
+    // and row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
+    float* const ring = reinterpret_cast<float*>(lds_all + SG::kStages * G::kKTile + wave * SG::kRingBytes);
+    uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
+    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
+    int ring_n = 0, stream_n = 0;  // wave-uniform
+    // (kt: the tile being worked on; a stream that fills faster than the tiles go by will not last: give up early)
+    auto flush = [&](int parity, int kt) {
+      for (int e0 = 0; e0 < ring_n; e0 += 64) {
+        const int e = e0 + lane;
+        const bool has = e < ring_n;
+        f32x4 w0 = {0.f, 0.f, 0.f, 0.f}, w1 = {0.f, 0.f, 0.f, 0.f};
+        uint32_t tag = 0u;
+        if (has) {
+          w0 = *reinterpret_cast<const f32x4*>(ring + e * 8);
+          w1 = *reinterpret_cast<const f32x4*>(ring + e * 8 + 4);
+          tag = ring_tag[e];
+        }
+        int c = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c += (w0[i] > 0.f ? 1 : 0) + (w1[i] > 0.f ? 1 : 0);
+        const int incl = wave_scan_i(c);
+        const int total_c = __builtin_amdgcn_readlane(incl, 63);
+        if (stream_n + total_c > SG::kListCap || (long long)(stream_n + total_c) * nt > (long long)SG::kListCap * (kt + 16)) {
+          if (lane == 0) s_giveup[parity] = 1u;
+        } else {
+          // producer lane = tag & 63: row (tag & 31), key half (tag >> 5) & 1; half block (tag >> 6) & 3 of tile tag >> 8
+          const uint32_t key0 = (tag >> 8) * kBN + ((tag >> 6) & 3u) * 16 + 4 * ((tag >> 5) & 1u);
+          const uint32_t rowbits = (tag & 31u) << 20;
+          uint2* dst = stream + stream_n + (incl - c);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float x = i < 4 ? w0[i & 3] : w1[i & 3];
+            if (x > 0.f) {
+              *dst = uint2{__builtin_bit_cast(uint32_t, x), (key0 + 8 * (i >> 2) + (i & 3)) | rowbits};
+              ++dst;
+            }
+          }
+          stream_n += total_c;
+        }
+      }
+      ring_n = 0;
+    };
+    // the lanes of `m` (those of them for which `mine` holds put their half block) take consecutive ring slots
+    auto put = [&](unsigned long long m, bool mine, const f32x16& s, int first, uint32_t tag, int kt) {
+      const int c = __builtin_popcountll(m);
+      if (ring_n + c > SG::kRing) flush(kt & 1, kt);
+      if (mine) {
+        const int slot = ring_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        f32x4 w0 = {s[first], s[first + 1], s[first + 2], s[first + 3]};
+        f32x4 w1 = {s[first + 4], s[first + 5], s[first + 6], s[first + 7]};
+        *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
+        *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
+        ring_tag[slot] = (tag << 6) | (uint32_t)lane;
+      }
+      ring_n += c;
+    };
+    auto collect = [&](const f32x16& s, int first, float hmax, uint32_t tag, int kt) {
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(hmax > 0.f);
+      if (m != 0ull) {
+        if (__builtin_popcountll(m) <= SG::kRing) {
+          put(m, hmax > 0.f, s, first, tag, kt);
+        } else {  // more events than the ring holds at once (the first tiles of a sequence): in two halves
+          put(m & 0xffffffffull, hmax > 0.f && lane < 32, s, first, tag, kt);
+          put(m & ~0xffffffffull, hmax > 0.f && lane >= 32, s, first, tag, kt);
+        }
+      }
+    };
+    walk(std::integral_constant<int, SG::kStages>{}, std::integral_constant<int, G::kKTile>{}, std::integral_constant<int, kKPer>{}, issue_k, [&](int kt, const unsigned char* kt_lds) {
+      for_tile(kt, kt_lds, -lo_raw, [&](const f32x16& s0, const f32x16& s1) {
+        float h00 = s0[0], h01 = s0[8], h10 = s1[0], h11 = s1[8];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+          h00 = fmaxf(h00, s0[i]);
+          h01 = fmaxf(h01, s0[8 + i]);
+          h10 = fmaxf(h10, s1[i]);
+          h11 = fmaxf(h11, s1[8 + i]);
+        }
+        collect(s0, 0, h00, (uint32_t)(kt * 4 + 0), kt);
+        collect(s0, 8, h01, (uint32_t)(kt * 4 + 1), kt);
+        collect(s1, 0, h10, (uint32_t)(kt * 4 + 2), kt);
+        collect(s1, 8, h11, (uint32_t)(kt * 4 + 3), kt);
+      });
+    });
+    flush(0, nt);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
+    __syncthreads();                      // every wave has left the K tiles: LDS becomes the lists
+    if (s_giveup[0] | s_giveup[1]) {
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(&p.queue[kCtrlFlagged], 1u);
+        atomicAdd(hint, 1u);
+        atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
+      }
+      continue;
+    }
+
+    // ---- the wave's stream -> per-row lists in its share of LDS (a counting sort by row) ----------------------------
+    unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
+    float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap scores minus the threshold
+    uint16_t* const lkey = reinterpret_cast<uint16_t*>(wave_lds + SG::kListCap * 4);         // their keys
+    uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 6);     // 32 counters
+    uint32_t* const row_start = row_cnt + 32;                                                // 33 offsets
+    if (lane < 32) row_cnt[lane] = 0u;
+    {
+      constexpr int kPer = (SG::kListCap + 63) / 64;
+      uint2 ent[kPer];
+      uint32_t pos[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        ent[j] = uint2{0u, 0u};
+        if (e < stream_n) ent[j] = stream[e];
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        pos[j] = 0u;
+        if (e < stream_n) pos[j] = atomicAdd(&row_cnt[(ent[j].y >> 20) & 31u], 1u);
+      }
+      {
+        const int c = lane < 32 ? (int)row_cnt[lane] : 0;
+        const int incl = wave_scan_i(c);
+        if (lane < 32) row_start[lane] = (uint32_t)(incl - c);
+        if (lane == 31) row_start[32] = (uint32_t)incl;
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        if (e < stream_n) {
+          const uint32_t at = row_start[(ent[j].y >> 20) & 31u] + pos[j];
+          lval[at] = __builtin_bit_cast(float, ent[j].x);
+          lkey[at] = (uint16_t)(ent[j].y & 0xffffu);
+        }
+      }
+    }
+
+    // ---- per row: dP over the support, delta, dQ.  A group of D / 8 lanes per row, each lane 8 columns; the V and K
+    // rows of kDepth members of the support are in flight together.  delta is only known behind the last member, so
+    // the lanes keep A = sum u dP k and B = sum u k and form (A - delta B) / sqrt(D) at the end. ---------------------
+    {
+      constexpr int kLPR = D / 8;         // lanes per row
+      constexpr int kGroups = 64 / kLPR;  // rows in progress per wave
+      constexpr int kDepth = 4;
+      const int grp = lane / kLPR, col = lane % kLPR;
+      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
+      const unsigned char* krows = kglob + col * 16;
+      const unsigned char* dorows = reinterpret_cast<const unsigned char*>(p.dout) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
+      unsigned char* dqrows = reinterpret_cast<unsigned char*>(p.dq) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
+      for (int r0 = 0; r0 < 32; r0 += kGroups) {
+        const int r = r0 + grp;
+        const bool row_live = wave_row0 + r < L;
+        const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
+        float dov[8];  // the lane's eight columns of dO_i (rows past the valid length may hold anything: not read)
+        {
+          u32x4 raw = {0u, 0u, 0u, 0u};
+          if (row_live) raw = *reinterpret_cast<const u32x4*>(dorows + (size_t)r * (D * 2));
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            dov[2 * i] = unpack_lo<T>(raw[i]);
+            dov[2 * i + 1] = unpack_hi<T>(raw[i]);
+          }
+        }
+        float acc_a[8], acc_b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          acc_a[i] = 0.f;
+          acc_b[i] = 0.f;
+        }
+        float zsum = 0.f, usum = 0.f, udp = 0.f;
+        for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+          u32x4 vv[kDepth], kk[kDepth];
+          float val[kDepth];
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            val[j] = 0.f;
+            vv[j] = u32x4{0u, 0u, 0u, 0u};
+            kk[j] = u32x4{0u, 0u, 0u, 0u};
+            if (eb + j < e_hi) {
+              const uint32_t key = lkey[eb + j];
+              val[j] = lval[eb + j];
+              vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
+              kk[j] = *reinterpret_cast<const u32x4*>(krows + (size_t)key * (D * 2));
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            float part = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part = fmaf(dov[2 * i], unpack_lo<T>(vv[j][i]), fmaf(dov[2 * i + 1], unpack_hi<T>(vv[j][i]), part));
+            const float dp = group_sum<kLPR>(part);  // dO_i . v_j, in every lane of the group
+            float pr, u;
+            bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
+            zsum += pr;
+            usum += u;
+            udp = fmaf(u, dp, udp);
+            const float wa = u * dp;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float klo = unpack_lo<T>(kk[j][i]), khi = unpack_hi<T>(kk[j][i]);
+              acc_a[2 * i] = fmaf(wa, klo, acc_a[2 * i]);
+              acc_a[2 * i + 1] = fmaf(wa, khi, acc_a[2 * i + 1]);
+              acc_b[2 * i] = fmaf(u, klo, acc_b[2 * i]);
+              acc_b[2 * i + 1] = fmaf(u, khi, acc_b[2 * i + 1]);
+            }
+          }
+        }
+        const float delta = usum > 0.f ? udp / usum : 0.f;
+        if (wave_row0 + r < N) {
+          float g[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) g[i] = row_live ? p.sm_scale * (acc_a[i] - delta * acc_b[i]) : 0.f;
+          u32x4 w = {pack2<T>(g[0], g[1]), pack2<T>(g[2], g[3]), pack2<T>(g[4], g[5]), pack2<T>(g[6], g[7])};
+          *reinterpret_cast<u32x4*>(dqrows + (size_t)r * (D * 2)) = w;
+        }
+        if (row_live && col == 0) {
+          const size_t at = (size_t)(b * p.Hq + h) * N + wave_row0 + r;
+          p.delta[at] = delta;
+          p.zinv[at] = zsum > 0.f ? 1.f / zsum : 0.f;
+        }
+      }
+    }
+    if (tid == 0) {
+      *flag = 0;
+      if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
+        atomicAdd(hint + 1, 1u);
+        atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);
+        known_unit = b * p.Hkv + kvh;
+      }
+    }
+  }
+}
+
+
+// Workgroups to launch: as many as fit the device at once (each owns one stream slot), at most `max_slots`.
+template <typename T, int D, int AM> static int launch_attn_bwd_sparse_one(const AttnBwdParams& p, int max_slots, hipStream_t s) {
+  using SG = SparseGeo<T, D>;
+  auto kern = attn_bwd_dq_sparse_kernel<T, D, AM>;
+  static int per_cu = 0, n_cu = 0;  // (one device family per process: gfx950)
+  if (per_cu == 0) {
+    int dev = 0, blocks = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 2;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kern, SG::kThreads, 0) != hipSuccess || blocks <= 0) blocks = 1;
+    n_cu = prop.multiProcessorCount;
+    per_cu = blocks;
+  }
+  long long grid = (long long)per_cu * n_cu;
+  if (grid > max_slots) grid = max_slots;
+  grid = grid / 8 * 8;  // the same number of workgroups on every XCD
+  if (grid < 8) grid = 8;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(SG::kThreads), 0, s, p);
+  return 0;
+}
+
+template <typename T, int D> static int launch_attn_bwd_sparse(const AttnBwdParams& p, int am, int max_slots, hipStream_t s) {
+  if (am == ATT_15) return launch_attn_bwd_sparse_one<T, D, ATT_15>(p, max_slots, s);
+  if (am == ATT_2) return launch_attn_bwd_sparse_one<T, D, ATT_2>(p, max_slots, s);
+  return 2;
+}
+
+}  // namespace adsp

@@ -170,3 +170,52 @@ def test_padding_rows_may_hold_anything(sparse_switch):
         t[:, :, 150:] = float("nan")
     out = forward(q, k, v, varlen)[0]
     assert max_err(out, want) < 2e-2 and (out[:, :, 150:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D,lens,alpha,causal,version", [
+    (2, 4, 2, 512, 128, [512, 300], 1.5, True, 2),
+    (1, 4, 1, 2048, 128, [1999], 1.5, True, 2),
+    (2, 2, 2, 200, 64, [137, 200], 1.5, True, 2),
+    (1, 2, 2, 512, 64, None, 2.0, False, 1),
+    (2, 2, 2, 384, 128, [384, 129], 1.5, False, 1),
+])
+def test_sparse_and_dense_dq_agree_with_the_oracle(sparse_switch, dtype, B, Hq, Hkv, N, D, lens, alpha, causal, version):
+    """The backward's dQ comes from the rows' supports (sparse-support dQ kernel) or from the dense kernel
+    (ADSP_SPARSE=0); dK and dV always come from the dense kernel, which reads delta and 1 / sum p from whichever of the
+    two wrote them.  All three gradients against the oracle on both settings, dQ of the two against each other."""
+    q, k, v = qkv(B, Hq, Hkv, N, D, dtype, seed=N + D + 1, scale=2.0 if alpha == 2.0 else 1.0)
+    varlen = None if lens is None else torch.tensor(lens, dtype=torch.int32)
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(2)).to(dtype)
+    want = exact.dense_entmax_attention_grads(q, k, v, dout, alpha, causal, varlen)
+    grads = {}
+    for on in (True, False):
+        sparse_switch(on)
+        qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+        vl = None if varlen is None else varlen.to(DEV)
+        if version == 2:
+            out = A.adasplash_v2(qg, kg, vg, varlen=vl)
+        else:
+            out = A.adasplash_v1(qg, kg, vg, alpha=alpha, is_causal=causal, varlen=vl)
+        out.backward(dout.to(DEV))
+        grads[on] = (qg.grad, kg.grad, vg.grad)
+        for got, ref in zip(grads[on], want):
+            assert max_err(got, ref) < 4e-2
+    assert max_err(grads[True][0], grads[False][0].float().cpu()) < 4e-2
+    if lens is not None:
+        for b, l in enumerate(lens):
+            assert (grads[True][0][b, :, l:] == 0).all()
+
+
+def test_dense_supports_leave_dq_to_the_dense_kernel(sparse_switch):
+    """Flat scores: the sparse-support dQ kernel gives every row block up and the result is the dense kernel's."""
+    q, k, v = qkv(1, 4, 4, 1024, 64, torch.bfloat16, seed=3, scale=0.125)
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16)
+    grads = {}
+    for on in (True, False):
+        sparse_switch(on)
+        qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+        A.adasplash_v2(qg, kg, vg, niter=1).backward(dout.to(DEV))
+        grads[on] = (qg.grad, kg.grad, vg.grad)
+    for a, b in zip(grads[True], grads[False]):
+        assert torch.equal(a, b)
