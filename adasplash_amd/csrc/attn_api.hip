@@ -13,7 +13,7 @@ namespace adsp {
 #define ADSP_DECL_D(tag, d)                                                      \
   int launch_attn_fwd_##tag##_d##d##_m0(const AttnParams&, int, hipStream_t);   \
   int launch_attn_fwd_##tag##_d##d##_m1(const AttnParams&, int, hipStream_t);   \
-  int launch_attn_bwd_##tag##_d##d(const AttnBwdParams&, int, hipStream_t);
+  int launch_attn_bwd_##tag##_d##d(const AttnBwdParams&, int, int, hipStream_t);
 #define ADSP_DECL_TAG(tag) ADSP_DECL_D(tag, 16) ADSP_DECL_D(tag, 32) ADSP_DECL_D(tag, 64) ADSP_DECL_D(tag, 128) ADSP_DECL_D(tag, 256)
 ADSP_DECL_TAG(f32)
 ADSP_DECL_TAG(bf16)
@@ -24,13 +24,13 @@ int launch_attn_sparse_bf16_d128(const AttnParams&, int, int, hipStream_t);
 int launch_attn_sparse_f16_d64(const AttnParams&, int, int, hipStream_t);
 int launch_attn_sparse_f16_d128(const AttnParams&, int, int, hipStream_t);
 // attn_bwd_dq_sparse_kernel (attn_bwd_sparse_unit.hip): likewise
-int launch_attn_bwd_sparse_bf16_d64(const AttnBwdParams&, int, int, hipStream_t);
-int launch_attn_bwd_sparse_bf16_d128(const AttnBwdParams&, int, int, hipStream_t);
-int launch_attn_bwd_sparse_f16_d64(const AttnBwdParams&, int, int, hipStream_t);
-int launch_attn_bwd_sparse_f16_d128(const AttnBwdParams&, int, int, hipStream_t);
+int launch_attn_bwd_sparse_bf16_d64(const AttnBwdParams&, int, int, int, hipStream_t);
+int launch_attn_bwd_sparse_bf16_d128(const AttnBwdParams&, int, int, int, hipStream_t);
+int launch_attn_bwd_sparse_f16_d64(const AttnBwdParams&, int, int, int, hipStream_t);
+int launch_attn_bwd_sparse_f16_d128(const AttnBwdParams&, int, int, int, hipStream_t);
 
 typedef int (*attn_fwd_fn)(const AttnParams&, int, hipStream_t);
-typedef int (*attn_bwd_fn)(const AttnBwdParams&, int, hipStream_t);
+typedef int (*attn_bwd_fn)(const AttnBwdParams&, int, int, hipStream_t);
 #define ADSP_FWD_ROW(tag, d) {launch_attn_fwd_##tag##_d##d##_m0, launch_attn_fwd_##tag##_d##d##_m1}
 #define ADSP_FWD_TAG(tag) {ADSP_FWD_ROW(tag, 16), ADSP_FWD_ROW(tag, 32), ADSP_FWD_ROW(tag, 64), ADSP_FWD_ROW(tag, 128), ADSP_FWD_ROW(tag, 256)}
 #define ADSP_BWD_TAG(tag) {launch_attn_bwd_##tag##_d16, launch_attn_bwd_##tag##_d32, launch_attn_bwd_##tag##_d64, launch_attn_bwd_##tag##_d128, launch_attn_bwd_##tag##_d256}
@@ -408,8 +408,8 @@ namespace adsp {
 // head dims the sparse-support dQ kernel serves -- its work counters, per-row-block flags and candidate streams (the
 // forward's layout without the copy of K).
 struct BwdWorkspace {
-  size_t copies_bytes, queue_off, flags_off, events_off, total;
-  int slots;  // 0: no sparse-support kernel for these dimensions
+  size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, part_off, part_bytes, total;
+  int slots;  // 0: no sparse-support kernels for these dimensions
 };
 static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
   BwdWorkspace w = {};
@@ -424,9 +424,67 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     w.queue_off = align256(w.copies_bytes);
     w.flags_off = align256(w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8);
     w.events_off = align256(w.flags_off + (size_t)items * 4);
-    w.total = w.events_off + (size_t)slots * kSparseSlotBytes;
+    // the dK/dV kernel: control words and hint counters of its own, a flag per (K/V head, key block), and fp32
+    // partial rows of dK and dV per query head
+    w.queue2_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
+    w.kvflags_off = align256(w.queue2_off + 256 + ((size_t)B * Hkv + 1) * 8);
+    w.part_off = align256(w.kvflags_off + (size_t)B * Hkv * mblocks_of(N) * 4);
+    w.part_bytes = (size_t)B * Hq * N * D * 4;
+    w.total = w.part_off + 2 * w.part_bytes;
   }
   return w;
+}
+
+// Clears the control words, hint counters and key-block flags of the sparse-support dK/dV kernel; the K/V heads the
+// probe marked as dense (in the dQ kernel's hint words) stay marked.
+__global__ __launch_bounds__(256) void bwd_ctrl_clear_kernel(uint32_t* ctrl2, const uint32_t* hints1, int units, int32_t* kv_flags,
+                                                            long long n_flags) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < 10) ctrl2[i] = 0u;
+  if (i < units) {
+    ctrl2[64 + 2 * i] = hints1[2 * i] >= (1u << 20) ? (1u << 20) : 0u;
+    ctrl2[64 + 2 * i + 1] = 0u;
+  }
+  if (i < 2) ctrl2[64 + 2 * units + i] = 0u;
+  for (long long j = i; j < n_flags; j += (long long)gridDim.x * 256) kv_flags[j] = 0;
+}
+
+// dK, dV = sum over the query heads of a K/V head of the sparse-support kernel's fp32 partial rows; key blocks left to
+// attn_bwd_dkdv_kernel are skipped (that kernel writes them).  A thread adds up 8 columns of one key row.
+typedef float reduce_f32x4 __attribute__((ext_vector_type(4)));
+template <typename T>
+__global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restrict__ dk_part, const float* __restrict__ dv_part,
+                                                         void* dk, void* dv, const int32_t* kv_flags, const uint32_t* ctrl2,
+                                                         int B, int Hq, int Hkv, int N, int D) {
+  if (ctrl2[kCtrlAllDense] != 0u) return;
+  const int per_row = D / 8;
+  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long long)B * Hkv * N * per_row) return;
+  const int c = (int)(id % per_row);
+  const long long rg = id / per_row;
+  const int row = (int)(rg % N), bkv = (int)(rg / N);
+  if (kv_flags[(size_t)bkv * ((N + kMaskRows - 1) / kMaskRows) + row / kMaskRows] != 0) return;
+  const int group = Hq / Hkv, b = bkv / Hkv, kvh = bkv % Hkv;
+  float sk[8], sv[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sk[i] = sv[i] = 0.f;
+  for (int g = 0; g < group; ++g) {
+    const size_t at = (((size_t)(b * Hq + kvh * group + g) * N) + row) * D + c * 8;
+    const reduce_f32x4 k0 = *reinterpret_cast<const reduce_f32x4*>(dk_part + at), k1 = *reinterpret_cast<const reduce_f32x4*>(dk_part + at + 4);
+    const reduce_f32x4 v0 = *reinterpret_cast<const reduce_f32x4*>(dv_part + at), v1 = *reinterpret_cast<const reduce_f32x4*>(dv_part + at + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sk[i] += k0[i];
+      sk[4 + i] += k1[i];
+      sv[i] += v0[i];
+      sv[4 + i] += v1[i];
+    }
+  }
+  const size_t out = (((size_t)bkv * N) + row) * D + c * 8;
+  const u32x4 wk = {pack2<T>(sk[0], sk[1]), pack2<T>(sk[2], sk[3]), pack2<T>(sk[4], sk[5]), pack2<T>(sk[6], sk[7])};
+  const u32x4 wv = {pack2<T>(sv[0], sv[1]), pack2<T>(sv[2], sv[3]), pack2<T>(sv[4], sv[5]), pack2<T>(sv[6], sv[7])};
+  *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(dk) + out) = wk;
+  *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(dv) + out) = wv;
 }
 }  // namespace adsp
 
@@ -481,29 +539,29 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   p.queue = nullptr;
   p.hints = nullptr;
   p.events = nullptr;
+  p.queue2 = nullptr;
+  p.hints2 = nullptr;
+  p.kv_flags = nullptr;
+  p.dk_part = nullptr;
+  p.dv_part = nullptr;
   const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
+  bool sparse = false;
+  BwdWorkspace w = {};
 
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
-    const BwdWorkspace w = bwd_workspace(B, Hq, Hkv, N, D, dtype);
+    w = bwd_workspace(B, Hq, Hkv, N, D, dtype);
     const size_t need = w.total;
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
     uint16_t* kt = (uint16_t*)workspace;
     uint16_t* qt = kt + (size_t)B * Hkv * D * p.Npad;
     uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
-    const unsigned gx = vt_layout_blocks(p.Npad, D);
-    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hkv)), dim3(256), 0, s, (const uint16_t*)k, kt, N, p.Npad, D,
-                       varlen, varlen_bits, Hkv, (const uint32_t*)nullptr);
-    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, qt, N, p.Npad, D,
-                       varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
-    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, dot, N, p.Npad,
-                       D, varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
     p.kt = kt;
     p.qt = qt;
     p.dot = dot;
     // Sparse-support dQ kernel first (alpha 1.5 / 2): it serves the row blocks whose supports are short and flags the
     // others for attn_bwd_dq_kernel below; the dK/dV kernel reads delta and 1 / sum p from whichever of the two wrote them.
-    const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
+    sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
     if (sparse) {
       unsigned char* ws = (unsigned char*)workspace;
       p.queue = (uint32_t*)(ws + w.queue_off);
@@ -526,16 +584,72 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
       int rc;
       if (dtype == ADSP_BF16) {
         hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, pp, D, am);
-        rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, w.slots, s);
+        rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, 0, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, 0, w.slots, s);
       } else {
         hipLaunchKernelGGL(attn_probe_kernel<f16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, pp, D, am);
-        rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, w.slots, s);
+        rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, 0, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, 0, w.slots, s);
       }
       if (rc != 0) return ADSP_ERR_LAUNCH;
     }
+    // the transposed copies serve the dense kernels only: that of k the dQ kernel (skipped when the sparse-support
+    // kernel left it nothing), those of q and dout the dK/dV kernel (made further down when the sparse path is taken)
+    const unsigned gx = vt_layout_blocks(p.Npad, D);
+    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hkv)), dim3(256), 0, s, (const uint16_t*)k, kt, N, p.Npad, D,
+                       varlen, varlen_bits, Hkv, (const uint32_t*)p.queue);
+    if (!sparse) {
+      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, qt, N, p.Npad, D,
+                         varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
+      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, dot, N, p.Npad,
+                         D, varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
+    }
   }
-  int rc = kBwdTable[dtype][head_dim_slot(D)](p, am, s);
-  if (rc != 0) return ADSP_ERR_LAUNCH;
+  if (!sparse) {
+    if (kBwdTable[dtype][head_dim_slot(D)](p, am, 3, s) != 0) return ADSP_ERR_LAUNCH;
+    return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
+  }
+  // dense dQ kernel on the row blocks the sparse one flagged (delta and 1 / sum p are complete behind it), then dK and
+  // dV: the sparse-support kernel per (key block, query head), the dense kernel on the key blocks it flagged, and the
+  // sum of the partial rows over the query heads of each K/V head
+  if (kBwdTable[dtype][head_dim_slot(D)](p, am, 1, s) != 0) return ADSP_ERR_LAUNCH;
+  {
+    unsigned char* ws = (unsigned char*)workspace;
+    p.queue2 = (uint32_t*)(ws + w.queue2_off);
+    p.hints2 = p.queue2 + 64;
+    p.kv_flags = (int32_t*)(ws + w.kvflags_off);
+    if (w.part_bytes) {
+      p.dk_part = (float*)(ws + w.part_off);
+      p.dv_part = (float*)(ws + w.part_off + w.part_bytes);
+    }
+    const long long n_flags = (long long)B * Hkv * mblocks_of(N);
+    long long clear_items = n_flags > (long long)B * Hkv ? n_flags : (long long)B * Hkv;  // (at least one thread per K/V head and per control word)
+    if (clear_items < 10) clear_items = 10;
+    long long clear_blocks = (clear_items + 255) / 256;
+    if (clear_blocks > 1024) clear_blocks = 1024;
+    hipLaunchKernelGGL(bwd_ctrl_clear_kernel, dim3((unsigned)clear_blocks), dim3(256), 0, s, p.queue2, (const uint32_t*)p.hints, B * Hkv,
+                       p.kv_flags, n_flags);
+    int rc;
+    if (dtype == ADSP_BF16) rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, 1, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, 1, w.slots, s);
+    else rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, 1, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, 1, w.slots, s);
+    if (rc != 0) return ADSP_ERR_LAUNCH;
+    {
+      const unsigned gx = vt_layout_blocks(p.Npad, D);
+      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, (uint16_t*)const_cast<void*>(p.qt), N, p.Npad, D,
+                         varlen, varlen_bits, Hq, (const uint32_t*)p.queue2);
+      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, (uint16_t*)const_cast<void*>(p.dot), N, p.Npad,
+                         D, varlen, varlen_bits, Hq, (const uint32_t*)p.queue2);
+    }
+    if (kBwdTable[dtype][head_dim_slot(D)](p, am, 2, s) != 0) return ADSP_ERR_LAUNCH;
+    if (w.part_bytes) {
+      const long long threads = (long long)B * Hkv * N * (D / 8);
+      const dim3 grid((unsigned)((threads + 255) / 256));
+      if (dtype == ADSP_BF16)
+        hipLaunchKernelGGL(dkdv_reduce_kernel<bf16_t>, grid, dim3(256), 0, s, (const float*)p.dk_part, (const float*)p.dv_part, dk, dv,
+                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, B, Hq, Hkv, N, D);
+      else
+        hipLaunchKernelGGL(dkdv_reduce_kernel<f16_t>, grid, dim3(256), 0, s, (const float*)p.dk_part, (const float*)p.dv_part, dk, dv,
+                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, B, Hq, Hkv, N, D);
+    }
+  }
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
 }
 

@@ -536,6 +536,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   if (!bwd_block_map(p.B * p.Hkv, (N + kBwdRows - 1) / kBwdRows, bkv, nblk)) return;
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int group = p.Hq / p.Hkv;
+  // behind the sparse-support dK/dV kernel: only the key blocks it flagged (all of them when it stepped aside)
+  if (p.kv_flags && p.queue2[kCtrlAllDense] == 0u &&
+      (p.queue2[kCtrlFlagged] == 0u || p.kv_flags[(size_t)bkv * ((N + kBwdRows - 1) / kBwdRows) + nblk] == 0))
+    return;
   const int L = bwd_seq_len(p, b);
   const int n0 = nblk * kBwdRows;
   const int wave_key0 = n0 + wave * 32;
@@ -807,18 +811,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   BT::store_rows(acc, p.sm_scale, stage, dk_rows, wave_key0, N, lane);
 }
 
-template <typename T, int D> static int launch_attn_bwd_d(const AttnBwdParams& p, int am, hipStream_t s) {
+// which: 1 = the dQ kernel, 2 = the dK/dV kernel, 3 = both, in that order
+template <typename T, int D> static int launch_attn_bwd_d(const AttnBwdParams& p, int am, int which, hipStream_t s) {
   const long long nq = (p.N + kBwdRows - 1) / kBwdRows;
   const dim3 gq((unsigned)(((long long)p.B * p.Hq * nq + 7) / 8 * 8)), gk((unsigned)(((long long)p.B * p.Hkv * nq + 7) / 8 * 8));
   if (am == ATT_15) {
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_15>), gq, dim3(256), 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_15>), gk, dim3(256), 0, s, p);
+    if (which & 1) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_15>), gq, dim3(256), 0, s, p);
+    if (which & 2) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_15>), gk, dim3(256), 0, s, p);
   } else if (am == ATT_2) {
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_2>), gq, dim3(256), 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_2>), gk, dim3(256), 0, s, p);
+    if (which & 1) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_2>), gq, dim3(256), 0, s, p);
+    if (which & 2) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_2>), gk, dim3(256), 0, s, p);
   } else {
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_GEN>), gq, dim3(256), 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_GEN>), gk, dim3(256), 0, s, p);
+    if (which & 1) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, ATT_GEN>), gq, dim3(256), 0, s, p);
+    if (which & 2) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, ATT_GEN>), gk, dim3(256), 0, s, p);
   }
   return 0;
 }

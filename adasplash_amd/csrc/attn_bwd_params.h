@@ -25,6 +25,13 @@ struct AttnBwdParams {
   uint32_t* queue;        // control words: work counters, flagged count, "every head dense"
   uint32_t* hints;        // two counters per K/V head and one pair over all heads
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
+  // the sparse-support dK/dV kernel: a control block of its own, one flag per (K/V head, key block), and fp32 partial
+  // rows [B, Hq, N, D] when a K/V head serves several query heads (null otherwise); the streams are shared
+  uint32_t* queue2;
+  uint32_t* hints2;
+  int32_t* kv_flags;  // [B, Hkv, n_mblk] 1 = key block left to attn_bwd_dkdv_kernel
+  float* dk_part;
+  float* dv_part;
 };
 
 }  // namespace adsp

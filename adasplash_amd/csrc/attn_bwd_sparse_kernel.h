@@ -19,6 +19,16 @@
 
 namespace adsp {
 
+// 4-byte global -> LDS copy per lane (lane i writes LDS bytes [4 i, 4 i + 4) after the wave-uniform base `lds`), the
+// global address given as a scalar base and a 32-bit byte offset per lane: dma16s of attn_kernel.h for single words
+__device__ __forceinline__ void dma4s(const void* gbase, uint32_t off, void* lds) {
+  const uint32_t base = (uint32_t)(uintptr_t)lds;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               :
+               : "v"(off), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(base))
+               : "memory");
+}
+
 // sum over a group of LANES (8 or 16) adjacent lanes, left in every lane of the group
 template <int LANES> __device__ __forceinline__ float group_sum(float x) {
   if constexpr (LANES == 16) {
@@ -503,11 +513,566 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 }
 
 
-// Workgroups to launch: as many as fit the device at once (each owns one stream slot), at most `max_slots`.
-template <typename T, int D, int AM> static int launch_attn_bwd_sparse_one(const AttnBwdParams& p, int max_slots, hipStream_t s) {
+// dK and dV from the keys' side of the same lists: the lane's "row" is a key, the tiles are rows of q of one query
+// head, and a score minus the *query's* threshold is positive exactly when the key lies in that query's support (the
+// thresholds of a tile's 64 queries arrive in LDS with the tile and are subtracted after the products).  The walk,
+// the ring, the stream and the counting sort are those of the dQ kernel with the roles swapped; the lists then hold,
+// per key, the queries that weight it.  A workgroup serves one (key block, query head).  The results are fp32
+// partial rows per query head that dkdv_reduce_kernel adds up over the heads of a K/V head.  The first key blocks of a
+// causal sequence lie in the supports of hundreds of queries each: when a wave's stream is half full the walk pauses,
+// the lists made so far are worked off into the partial rows, and the walk goes on.  A key block that any of its query
+// heads gives up all the same is flagged and computed, all heads, by attn_bwd_dkdv_kernel.
+template <typename T, int D, int AM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE_WAVES, ADSP_SPARSE_WAVES))) void attn_bwd_dkdv_sparse_kernel(AttnBwdParams p) {
+  using G = TileGeo<T, D>;
   using SG = SparseGeo<T, D>;
-  auto kern = attn_bwd_dq_sparse_kernel<T, D, AM>;
-  static int per_cu = 0, n_cu = 0;  // (one device family per process: gfx950)
+  using KS = Swz<G::kKRow>;
+  static_assert(G::k16, "16-bit element types only");
+  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  constexpr int NW = SG::kNW, BM = SG::kBM;
+  __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
+  __shared__ int s_item, s_skip;
+  // a lane ran out of event slots, or a wave out of list room.  Two words: the walks write the one of the tile's
+  // parity and read the other one behind the next barrier, so no wave can read a word another one is still setting
+  __shared__ uint32_t s_giveup[2];
+  __shared__ float s_tau[SG::kStages][kBN];  // thresholds of the tile's queries
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int N = p.N;
+  const int n_mblk = (N + BM - 1) / BM;
+  const int group = p.Hq / p.Hkv;
+  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
+  const long long per_xcd = (total + 7) / 8;
+  const float qs = p.qscale, inv_qs = 1.f / p.qscale;
+  constexpr int kKPer = (G::kKLoads + NW - 1) / NW;
+  constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
+  static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
+
+  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all row blocks
+    const int units = p.B * p.Hkv;
+    int unmarked = 0;
+    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints2[2 * u] < (1u << 20) ? 1 : 0;
+    if (__syncthreads_count(unmarked) == 0) {
+      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue2[kCtrlAllDense] = 1u;
+      return;
+    }
+  }
+  int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
+  int known_unit = -1;   // thread 0: the K/V head whose hint counters it has last seen (or set) as served
+  for (;;) {
+    // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
+    // of this loop they would stay live through both walks, and the walks have no registers to spare.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+    // tile DMA and fragment-read geometry (see attn_fwd_kernel)
+    const uint32_t koff = (uint32_t)((wave * 64 + lane) / KS::kC * G::kKRow + ((((wave * 64 + lane) % KS::kC) ^ KS::sw((wave * 64 + lane) / KS::kC)) << 4));
+    const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
+
+    __syncthreads();  // the previous row block is done with LDS and with s_item
+    if (tid == 0) {
+      int got = -1;
+      while (queues_tried < 8) {
+        const int x = ((int)(blockIdx.x & 7) + queues_tried) & 7;
+        const long long i = (long long)atomicAdd(&p.queue2[x], 1u);
+        const long long logical = (long long)x * per_xcd + i;
+        if (i < per_xcd && logical < total) {
+          got = (int)logical;
+          break;
+        }
+        ++queues_tried;
+      }
+      s_item = got;
+      s_skip = 0;
+      if (got >= 0) {  // the K/V head of the row block, as decoded below
+        int unit = got / (group * n_mblk);
+        const int units = p.B * p.Hkv;
+        if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
+        if (unit != known_unit) {
+          const uint32_t gave_up = __hip_atomic_load(p.hints2 + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t served = __hip_atomic_load(p.hints2 + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
+          const uint32_t all_gave_up = __hip_atomic_load(p.hints2 + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t all_served = __hip_atomic_load(p.hints2 + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // (the first key blocks of a causal sequence, which come first, collect the most queries and overflow even
+          // when the supports are short: only a long run of failures without a success says that the head is dense)
+          (void)all_gave_up;
+          (void)all_served;
+          s_skip = (gave_up >= (1u << 20) || (gave_up >= 32u && served == 0u)) ? 1 : 0;
+          if (served > 0u) known_unit = unit;
+        }
+      }
+      s_giveup[0] = 0u;
+      s_giveup[1] = 0u;
+    }
+    __syncthreads();
+    const int logical = s_item;
+    if (logical < 0) break;
+
+    // ---- row block -> (batch, kv head, row block, head in group), as in attn_fwd_kernel ---------------------
+    const int hg = logical % group;
+    const int mi = (logical / group) % n_mblk;
+    int bkv = logical / (group * n_mblk);
+    {
+      const int units = p.B * p.Hkv;
+      if (units % 8 == 0) bkv = (bkv % (units / 8)) * 8 + bkv / (units / 8);
+    }
+    const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
+    const int h = kvh * group + hg;
+    const int mblk = mi;  // key block: with a causal mask the first ones see the most queries
+    const int m0 = mblk * BM;
+    int L = N;
+    if (p.varlen) {
+      long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
+      L = (int)(l < 0 ? 0 : (l > N ? N : l));
+    }
+    // a key block that any query head gives up goes to attn_bwd_dkdv_kernel with all its heads
+    int32_t* const flag = p.kv_flags + ((size_t)(b * p.Hkv + kvh) * n_mblk + mblk);
+    // Row blocks of one K/V head tend to share their fate: once a few of them were given up and none succeeded, the
+    // rest go to the dense kernel unseen (a hint only: thread 0 read the counters, without any ordering, above).
+    uint32_t* const hint = p.hints2 + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
+    const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
+    const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
+    const int qi = m0 + wave * 32 + lq;
+
+    if (m0 >= L) {  // key block entirely inside the padding: zero gradient (nothing else writes these rows)
+      const int rows = (N - m0) < BM ? (N - m0) : BM;
+      float* o0 = p.dk_part + qo_base + (size_t)m0 * D;
+      float* o1 = p.dv_part + qo_base + (size_t)m0 * D;
+      for (int i = tid; i < rows * D; i += SG::kThreads) {
+        o0[i] = 0.f;
+        o1[i] = 0.f;
+      }
+      continue;
+    }
+
+    if (s_skip) {
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(&p.queue2[kCtrlFlagged], 1u);
+      }
+      continue;
+    }
+    // here the lane's "row" is a key (qi: its index) and the tiles hold queries: with a causal mask the tiles from the
+    // key block's first key on, else all of them
+    const int kt_first = p.causal ? m0 / kBN : 0;
+    const int nt = (L + kBN - 1) / kBN - kt_first;
+    const int lo_lim = p.causal ? qi : 0;  // first query that sees the lane's key
+    const int wave_row0 = m0 + wave * 32;
+    const bool live = qi < L;
+
+    // ---- K fragments of the lane's key; keys past the valid length are zero and collect nothing ------------------
+    const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.k) + kv_base + (size_t)(live ? qi : 0) * D;
+    uint32_t qf[G::kQRegs];  // (loaded at the start of every part of the walk: not kept through the list phases)
+    const float* const tau_rows = p.taus + (size_t)(b * p.Hq + h) * N;
+
+    // the tiles are rows of q of the item's query head; wave 0 also brings the thresholds of the tile's 64 queries
+    const unsigned char* kglob = reinterpret_cast<const unsigned char*>(p.q) + qo_base * 2;
+    auto issue_k = [&](unsigned char* lds, int cur) {
+      const int kt = kt_first + cur;
+      if (wave == 0) {
+        const int stage_i = (int)((lds - lds_all) / G::kKTile);
+        int gi = kt * kBN + lane;
+        gi = gi < N ? gi : N - 1;
+        dma4s(uniform_ptr(tau_rows), (uint32_t)gi * 4u, &s_tau[stage_i][0]);
+      }
+      const unsigned char* base = uniform_ptr(kglob + (size_t)kt * G::kKTile);
+      if ((kt + 1) * kBN <= N) {
+#pragma unroll
+        for (int j0 = 0; j0 < kKPer; ++j0) dma16s(base + j0 * (NW * 1024), koff, lds + (j0 * NW + wave) * 1024);
+      } else {  // the last tile sticks out of the tensor: rows past the end are masked later, any valid row will do
+        const unsigned char* g = uniform_ptr(kglob);
+        const int row0 = (int)(koff / G::kKRow);
+        const uint32_t coff = koff % G::kKRow;
+#pragma unroll
+        for (int j0 = 0; j0 < kKPer; ++j0) {
+          int gk = kt * kBN + row0 + j0 * (NW * 64 / KS::kC);
+          gk = gk < N ? gk : N - 1;
+          dma16s(g, (uint32_t)gk * (uint32_t)G::kKRow + coff, lds + (j0 * NW + wave) * 1024);
+        }
+      }
+    };
+    // body(kt, tile) over all key tiles of the row block; stops when a lane gave up.  The K tiles go through a ring of
+    // kStages LDS buffers: the load of tile t + kStages - 1 is issued behind the barrier that opens tile t (every wave
+    // is done with tile t - 1, whose buffer it takes) and has kStages - 1 tile times to arrive.
+    // (stages_c, tile_c, per_c: the ring's depth, the bytes of a tile and the loads per wave and tile, as constants)
+    // Here the walk starts at tile `first` and returns the tile it stopped in front of (nt: all done): a wave whose stream
+    // is half full asks for a break, the lists made so far are worked off, and the walk goes on from there.
+    auto walk = [&](int first, auto stages_c, auto tile_c, auto per_c, auto&& issue, auto&& body) -> int {
+      constexpr int kStages = decltype(stages_c)::value, kTile = decltype(tile_c)::value, kPer = decltype(per_c)::value;
+      __syncthreads();
+#pragma unroll
+      for (int s = 0; s < kStages - 1; ++s)
+        if (first + s < nt) issue(lds_all + s * kTile, first + s);
+      int stage = 0;  // buffer of tile cur
+      int cur = first;
+      for (; cur < nt; ++cur) {
+        // this wave's share of tile cur has landed: everything but the loads issued after it (those of the tiles in
+        // between; stores issued after it only make the wait longer than needed)
+        if (cur + kStages - 1 <= nt) {
+          if constexpr (kStages == 2) __builtin_amdgcn_s_waitcnt(0x0f70);
+          else __builtin_amdgcn_s_waitcnt(0x0f70 | ((kStages - 2) * kPer));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);  // the last tiles: nothing was issued behind them
+        }
+        __syncthreads();
+        if (cur > first && s_giveup[(cur + 1) & 1]) break;  // set while the previous tile was worked on
+        const int pre = cur + kStages - 1;
+        if (pre < nt) issue(lds_all + (stage == 0 ? kStages - 1 : stage - 1) * kTile, pre);
+        __builtin_amdgcn_sched_barrier(0);
+        body(cur, lds_all + stage * kTile);
+        stage = stage + 1 == kStages ? 0 : stage + 1;
+      }
+      return cur;
+    };
+    // S^T of one tile (two 32-key blocks), accumulators preloaded with `init`; f(s0, s1) unless no row of the wave
+    // sees the tile.  Scores past a row's last valid key are -inf.
+    auto for_tile = [&](int kt, const unsigned char* kt_lds, auto&& f) {
+      if (p.causal && kt * kBN + kBN - 1 < wave_row0) return;  // every query of the tile lies before the wave's keys
+      const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN < wave_row0 + 31);
+      f32x16 s0, s1;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s0[i] = 0.f;
+        s1[i] = 0.f;
+      }
+      uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k_lane;
+      asm volatile("" : "+v"(ka));
+      u32x4 a0[D / 16], a1[D / 16];
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a0[ks] = lds_read16(ka ^ (ks << 5));
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) a1[ks] = lds_read16(ka ^ (ks << 5), 32 * G::kKRow);
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s0 = mfma_16bit<T>(a0[ks], bq, s0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 bq = {qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]};
+        s1 = mfma_16bit<T>(a1[ks], bq, s1);
+      }
+      // the order of issue: four fragment reads ahead of the first product, then one read behind every product
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * (D / 16) - 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      {  // minus the queries' thresholds (raw units): what is left positive is a member of that query's support
+        const float* tq = &s_tau[(int)((kt_lds - lds_all) / G::kKTile)][4 * lh];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const f32x4 t0 = *reinterpret_cast<const f32x4*>(tq + 8 * g4), t1 = *reinterpret_cast<const f32x4*>(tq + 32 + 8 * g4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            s0[4 * g4 + e] = fmaf(t0[e], -inv_qs, s0[4 * g4 + e]);
+            s1[4 * g4 + e] = fmaf(t1[e], -inv_qs, s1[4 * g4 + e]);
+          }
+        }
+      }
+      if (need_mask) {  // queries past the sequence's end (their thresholds may hold anything) or before the lane's key
+        const int jb = kt * kBN + 4 * lh;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int i0 = jb + 8 * (i >> 2) + (i & 3), i1 = i0 + 32;
+          s0[i] = (i0 < L && i0 >= lo_lim) ? s0[i] : -INFINITY;
+          s1[i] = (i1 < L && i1 >= lo_lim) ? s1[i] : -INFINITY;
+        }
+      }
+      f(s0, s1);
+    };
+
+    // ---- the walk: collect the scores above the threshold ---------------------------------------------------------
+    // A lane whose eight scores of a 16-key half block have a positive maximum puts them, with a tag, into the wave's
+    // ring in LDS (slots are handed out with a ballot: no atomics).  When the ring is full the wave empties it, one
+    // event per lane: the positive entries go to the wave's candidate stream in global memory as (score - threshold, key
+    // and row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
+    float* const ring = reinterpret_cast<float*>(lds_all + SG::kStages * G::kKTile + wave * SG::kRingBytes);
+    uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
+    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
+    int ring_n = 0, stream_n = 0;  // wave-uniform
+    auto flush = [&](int parity, int kt) {
+      for (int e0 = 0; e0 < ring_n; e0 += 64) {
+        const int e = e0 + lane;
+        const bool has = e < ring_n;
+        f32x4 w0 = {0.f, 0.f, 0.f, 0.f}, w1 = {0.f, 0.f, 0.f, 0.f};
+        uint32_t tag = 0u;
+        if (has) {
+          w0 = *reinterpret_cast<const f32x4*>(ring + e * 8);
+          w1 = *reinterpret_cast<const f32x4*>(ring + e * 8 + 4);
+          tag = ring_tag[e];
+        }
+        int c = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c += (w0[i] > 0.f ? 1 : 0) + (w1[i] > 0.f ? 1 : 0);
+        const int incl = wave_scan_i(c);
+        const int total_c = __builtin_amdgcn_readlane(incl, 63);
+        // (no projection here: a key's queries thin out along the walk, the first tiles bring most of its members)
+        if (stream_n + total_c > SG::kListCap) {
+          if (lane == 0) atomicOr(&s_giveup[parity], 1u);  // bit 0: give the key block up
+        } else {
+          // producer lane = tag & 63: row (tag & 31), key half (tag >> 5) & 1; half block (tag >> 6) & 3 of tile tag >> 8
+          const uint32_t key0 = (tag >> 8) * kBN + ((tag >> 6) & 3u) * 16 + 4 * ((tag >> 5) & 1u);
+          const uint32_t rowbits = (tag & 31u) << 20;
+          uint2* dst = stream + stream_n + (incl - c);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float x = i < 4 ? w0[i & 3] : w1[i & 3];
+            if (x > 0.f) {
+              *dst = uint2{__builtin_bit_cast(uint32_t, x), (key0 + 8 * (i >> 2) + (i & 3)) | rowbits};
+              ++dst;
+            }
+          }
+          stream_n += total_c;
+          if (stream_n > SG::kListCap / 2 && lane == 0) atomicOr(&s_giveup[parity], 2u);  // bit 1: break the walk here
+        }
+      }
+      ring_n = 0;
+    };
+    // the lanes of `m` (those of them for which `mine` holds put their half block) take consecutive ring slots
+    auto put = [&](unsigned long long m, bool mine, const f32x16& s, int first, uint32_t tag, int kt) {
+      const int c = __builtin_popcountll(m);
+      if (ring_n + c > SG::kRing) flush(kt & 1, kt);
+      if (mine) {
+        const int slot = ring_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        f32x4 w0 = {s[first], s[first + 1], s[first + 2], s[first + 3]};
+        f32x4 w1 = {s[first + 4], s[first + 5], s[first + 6], s[first + 7]};
+        *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
+        *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
+        ring_tag[slot] = (tag << 6) | (uint32_t)lane;
+      }
+      ring_n += c;
+    };
+    auto collect = [&](const f32x16& s, int first, float hmax, uint32_t tag, int kt) {
+      const bool mine = hmax > 0.f && live;
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(mine);
+      if (m != 0ull) {
+        if (__builtin_popcountll(m) <= SG::kRing) {
+          put(m, mine, s, first, tag, kt);
+        } else {  // more events than the ring holds at once: in two halves
+          put(m & 0xffffffffull, mine && lane < 32, s, first, tag, kt);
+          put(m & ~0xffffffffull, mine && lane >= 32, s, first, tag, kt);
+        }
+      }
+    };
+    int done = 0;           // tiles of the item walked so far
+    bool gave_up = false;
+    for (int seg = 0;; ++seg) {
+    ring_n = 0;
+    stream_n = 0;
+    {
+      const uint16_t* krow = qrow;
+      asm volatile("" : "+v"(krow));  // (keeps the loads inside the loop)
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(krow + ks * 16 + 8 * lh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = live ? raw[e] : 0u;
+      }
+    }
+    done = walk(done, std::integral_constant<int, SG::kStages>{}, std::integral_constant<int, G::kKTile>{}, std::integral_constant<int, kKPer>{}, issue_k, [&](int cur, const unsigned char* kt_lds) {
+      const int kt = kt_first + cur;
+      for_tile(kt, kt_lds, [&](const f32x16& s0, const f32x16& s1) {
+        float h00 = s0[0], h01 = s0[8], h10 = s1[0], h11 = s1[8];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+          h00 = fmaxf(h00, s0[i]);
+          h01 = fmaxf(h01, s0[8 + i]);
+          h10 = fmaxf(h10, s1[i]);
+          h11 = fmaxf(h11, s1[8 + i]);
+        }
+        collect(s0, 0, h00, (uint32_t)(kt * 4 + 0), kt);
+        collect(s0, 8, h01, (uint32_t)(kt * 4 + 1), kt);
+        collect(s1, 0, h10, (uint32_t)(kt * 4 + 2), kt);
+        collect(s1, 8, h11, (uint32_t)(kt * 4 + 3), kt);
+      });
+    });
+    flush(0, kt_first + done);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
+    __syncthreads();                      // every wave has left the K tiles: LDS becomes the lists
+    if ((s_giveup[0] | s_giveup[1]) & 1u) {
+      gave_up = true;
+      break;
+    }
+
+    // ---- the wave's stream -> per-row lists in its share of LDS (a counting sort by row) ----------------------------
+    unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
+    float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap scores minus the threshold
+    uint16_t* const lkey = reinterpret_cast<uint16_t*>(wave_lds + SG::kListCap * 4);         // their keys
+    uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 6);     // 32 counters
+    uint32_t* const row_start = row_cnt + 32;                                                // 33 offsets
+    if (lane < 32) row_cnt[lane] = 0u;
+    {
+      constexpr int kPer = (SG::kListCap + 63) / 64;
+      uint2 ent[kPer];
+      uint32_t pos[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        ent[j] = uint2{0u, 0u};
+        if (e < stream_n) ent[j] = stream[e];
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        pos[j] = 0u;
+        if (e < stream_n) pos[j] = atomicAdd(&row_cnt[(ent[j].y >> 20) & 31u], 1u);
+      }
+      {
+        const int c = lane < 32 ? (int)row_cnt[lane] : 0;
+        const int incl = wave_scan_i(c);
+        if (lane < 32) row_start[lane] = (uint32_t)(incl - c);
+        if (lane == 31) row_start[32] = (uint32_t)incl;
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int e = j * 64 + lane;
+        if (e < stream_n) {
+          const uint32_t at = row_start[(ent[j].y >> 20) & 31u] + pos[j];
+          lval[at] = __builtin_bit_cast(float, ent[j].x);
+          lkey[at] = (uint16_t)(ent[j].y & 0xffffu);
+        }
+      }
+    }
+
+    // ---- per key: its list holds the queries (of this head) in whose support it lies, with score minus threshold.
+    // A group of D / 8 lanes per key, each lane 8 columns of v_j; per member it fetches its 16 bytes of dO_i and q_i and
+    // the row's delta_i and 1 / sum p (written by the dQ kernels), forms dP_ij = dO_i . v_j across the group and adds
+    // p_ij / sum p * dO_i to dV_j and u_ij (dP_ij - delta_i) * q_i to dK_j. ---------------------------------------------
+    {
+      constexpr int kLPR = D / 8;         // lanes per key
+      constexpr int kGroups = 64 / kLPR;  // keys in progress per wave
+      constexpr int kDepth = 4;
+      const int grp = lane / kLPR, col = lane % kLPR;
+      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
+      const unsigned char* qrows = kglob + col * 16;
+      const unsigned char* dorows = reinterpret_cast<const unsigned char*>(p.dout) + qo_base * 2 + col * 16;
+      const float* const delta_rows = p.delta + (size_t)(b * p.Hq + h) * N;
+      const float* const zinv_rows = p.zinv + (size_t)(b * p.Hq + h) * N;
+      for (int r0 = 0; r0 < 32; r0 += kGroups) {
+        const int r = r0 + grp;
+        const int key = wave_row0 + r;
+        const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
+        float vj[8];
+        {
+          u32x4 raw = {0u, 0u, 0u, 0u};
+          if (key < L) raw = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            vj[2 * i] = unpack_lo<T>(raw[i]);
+            vj[2 * i + 1] = unpack_hi<T>(raw[i]);
+          }
+        }
+        float acc_v[8], acc_k[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          acc_v[i] = 0.f;
+          acc_k[i] = 0.f;
+        }
+        for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+          u32x4 dd[kDepth], qq[kDepth];
+          float val[kDepth], dl[kDepth], zi[kDepth];
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            val[j] = 0.f;
+            dl[j] = 0.f;
+            zi[j] = 0.f;
+            dd[j] = u32x4{0u, 0u, 0u, 0u};
+            qq[j] = u32x4{0u, 0u, 0u, 0u};
+            if (eb + j < e_hi) {
+              const uint32_t qidx = lkey[eb + j];
+              val[j] = lval[eb + j];
+              dd[j] = *reinterpret_cast<const u32x4*>(dorows + (size_t)qidx * (D * 2));
+              qq[j] = *reinterpret_cast<const u32x4*>(qrows + (size_t)qidx * (D * 2));
+              dl[j] = delta_rows[qidx];
+              zi[j] = zinv_rows[qidx];
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            float dof[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              dof[2 * i] = unpack_lo<T>(dd[j][i]);
+              dof[2 * i + 1] = unpack_hi<T>(dd[j][i]);
+            }
+            float part = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part = fmaf(dof[i], vj[i], part);
+            const float dp = group_sum<kLPR>(part);  // dO_i . v_j, in every lane of the group
+            float pr, u;
+            bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
+            const float ph = pr * zi[j], dx = u * (dp - dl[j]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              acc_v[2 * i] = fmaf(ph, dof[2 * i], acc_v[2 * i]);
+              acc_v[2 * i + 1] = fmaf(ph, dof[2 * i + 1], acc_v[2 * i + 1]);
+              acc_k[2 * i] = fmaf(dx, unpack_lo<T>(qq[j][i]), acc_k[2 * i]);
+              acc_k[2 * i + 1] = fmaf(dx, unpack_hi<T>(qq[j][i]), acc_k[2 * i + 1]);
+            }
+          }
+        }
+        if (key < N) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc_k[i] *= p.sm_scale;
+          // fp32 partial rows of this query head (dkdv_reduce_kernel adds up the heads of a K/V head); a later part of
+          // the walk adds to what the earlier ones stored
+          float* o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
+          float* o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+          if (seg > 0) {
+            const f32x4 k0 = *reinterpret_cast<const f32x4*>(o0), k1 = *reinterpret_cast<const f32x4*>(o0 + 4);
+            const f32x4 v0 = *reinterpret_cast<const f32x4*>(o1), v1 = *reinterpret_cast<const f32x4*>(o1 + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              acc_k[i] += k0[i];
+              acc_k[4 + i] += k1[i];
+              acc_v[i] += v0[i];
+              acc_v[4 + i] += v1[i];
+            }
+          }
+          *reinterpret_cast<f32x4*>(o0) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
+          *reinterpret_cast<f32x4*>(o0 + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
+          *reinterpret_cast<f32x4*>(o1) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
+          *reinterpret_cast<f32x4*>(o1 + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+        }
+      }
+    }
+    if (done >= nt) break;
+    __syncthreads();  // every wave is done with its lists: the walk takes the tiles' room back
+    if (tid == 0) {
+      s_giveup[0] = 0u;
+      s_giveup[1] = 0u;
+    }
+    }  // (parts of the walk)
+    if (gave_up) {
+      if (tid == 0) {
+        *flag = 1;
+        atomicAdd(&p.queue2[kCtrlFlagged], 1u);
+        atomicAdd(hint, 1u);
+        atomicAdd(p.hints2 + 2 * p.B * p.Hkv, 1u);
+      }
+      continue;
+    }
+    if (tid == 0) {
+      if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
+        atomicAdd(hint + 1, 1u);
+        atomicAdd(p.hints2 + 2 * p.B * p.Hkv + 1, 1u);
+        known_unit = b * p.Hkv + kvh;
+      }
+    }
+  }
+}
+
+
+
+// Workgroups to launch: as many as fit the device at once (each owns one stream slot), at most `max_slots`.
+template <typename T, int D, int AM, bool kKeys> static int launch_attn_bwd_sparse_one(const AttnBwdParams& p, int max_slots, hipStream_t s) {
+  using SG = SparseGeo<T, D>;
+  auto kern = kKeys ? attn_bwd_dkdv_sparse_kernel<T, D, AM> : attn_bwd_dq_sparse_kernel<T, D, AM>;
+  static int per_cu = 0, n_cu = 0;  // (one device family per process: gfx950; one pair per instantiation)
   if (per_cu == 0) {
     int dev = 0, blocks = 0;
     hipDeviceProp_t prop;
@@ -524,9 +1089,10 @@ template <typename T, int D, int AM> static int launch_attn_bwd_sparse_one(const
   return 0;
 }
 
-template <typename T, int D> static int launch_attn_bwd_sparse(const AttnBwdParams& p, int am, int max_slots, hipStream_t s) {
-  if (am == ATT_15) return launch_attn_bwd_sparse_one<T, D, ATT_15>(p, max_slots, s);
-  if (am == ATT_2) return launch_attn_bwd_sparse_one<T, D, ATT_2>(p, max_slots, s);
+// keys = 0: the dQ kernel, 1: the dK/dV kernel
+template <typename T, int D> static int launch_attn_bwd_sparse(const AttnBwdParams& p, int am, int keys, int max_slots, hipStream_t s) {
+  if (am == ATT_15) return keys ? launch_attn_bwd_sparse_one<T, D, ATT_15, true>(p, max_slots, s) : launch_attn_bwd_sparse_one<T, D, ATT_15, false>(p, max_slots, s);
+  if (am == ATT_2) return keys ? launch_attn_bwd_sparse_one<T, D, ATT_2, true>(p, max_slots, s) : launch_attn_bwd_sparse_one<T, D, ATT_2, false>(p, max_slots, s);
   return 2;
 }
 

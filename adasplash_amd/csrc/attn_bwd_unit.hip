@@ -6,5 +6,5 @@
 #define ADSP_CAT(a, b) ADSP_CAT_(a, b)
 
 namespace adsp {
-int ADSP_CAT(ADSP_TAG, ADSP_D)(const AttnBwdParams& p, int am, hipStream_t s) { return launch_attn_bwd_d<ADSP_T, ADSP_D>(p, am, s); }
+int ADSP_CAT(ADSP_TAG, ADSP_D)(const AttnBwdParams& p, int am, int which, hipStream_t s) { return launch_attn_bwd_d<ADSP_T, ADSP_D>(p, am, which, s); }
 }  // namespace adsp

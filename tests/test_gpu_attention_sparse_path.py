@@ -207,15 +207,20 @@ def test_sparse_and_dense_dq_agree_with_the_oracle(sparse_switch, dtype, B, Hq, 
             assert (grads[True][0][b, :, l:] == 0).all()
 
 
-def test_dense_supports_leave_dq_to_the_dense_kernel(sparse_switch):
-    """Flat scores: the sparse-support dQ kernel gives every row block up and the result is the dense kernel's."""
+def test_dense_supports_go_back_to_the_dense_backward_kernels(sparse_switch):
+    """Flat scores: the sparse-support backward kernels give up the row blocks and key blocks whose lists overflow
+    (most of them; the last key blocks, which few queries see, may still fit) and the dense kernels redo those.  The
+    result agrees with the dense kernels' alone and with the oracle."""
     q, k, v = qkv(1, 4, 4, 1024, 64, torch.bfloat16, seed=3, scale=0.125)
     dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16)
+    want = exact.dense_entmax_attention_grads(q, k, v, dout, 1.5, True, None)
     grads = {}
     for on in (True, False):
         sparse_switch(on)
         qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
-        A.adasplash_v2(qg, kg, vg, niter=1).backward(dout.to(DEV))
+        A.adasplash_v2(qg, kg, vg, niter=10).backward(dout.to(DEV))
         grads[on] = (qg.grad, kg.grad, vg.grad)
+        for got, ref in zip(grads[on], want):
+            assert max_err(got, ref) < 4e-2
     for a, b in zip(grads[True], grads[False]):
-        assert torch.equal(a, b)
+        assert max_err(a, b.float().cpu()) < 4e-2
