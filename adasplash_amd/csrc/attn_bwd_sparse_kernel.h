@@ -609,7 +609,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     const int logical = s_item;
     if (logical < 0) break;
 
-    // ---- row block -> (batch, kv head, row block, head in group), as in attn_fwd_kernel ---------------------
+    // ---- item -> (batch, kv head, key block, head in group), in the order of the dQ kernel's row blocks ---------
     const int hg = logical % group;
     const int mi = (logical / group) % n_mblk;
     int bkv = logical / (group * n_mblk);
@@ -628,8 +628,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     }
     // a key block that any query head gives up goes to attn_bwd_dkdv_kernel with all its heads
     int32_t* const flag = p.kv_flags + ((size_t)(b * p.Hkv + kvh) * n_mblk + mblk);
-    // Row blocks of one K/V head tend to share their fate: once a few of them were given up and none succeeded, the
-    // rest go to the dense kernel unseen (a hint only: thread 0 read the counters, without any ordering, above).
+    // the K/V head's hint counters (thread 0 read them, without any ordering, above)
     uint32_t* const hint = p.hints2 + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
     const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
     const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
@@ -692,7 +691,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
     };
-    // body(kt, tile) over all key tiles of the row block; stops when a lane gave up.  The K tiles go through a ring of
+    // body(tile index, tile) over the query tiles of the item; stops when a lane gave up or asked for a break.  The tiles go through a ring of
     // kStages LDS buffers: the load of tile t + kStages - 1 is issued behind the barrier that opens tile t (every wave
     // is done with tile t - 1, whose buffer it takes) and has kStages - 1 tile times to arrive.
     // (stages_c, tile_c, per_c: the ring's depth, the bytes of a tile and the loads per wave and tile, as constants)
@@ -725,8 +724,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
       return cur;
     };
-    // S^T of one tile (two 32-key blocks), accumulators preloaded with `init`; f(s0, s1) unless no row of the wave
-    // sees the tile.  Scores past a row's last valid key are -inf.
+    // scores of one tile (two blocks of 32 queries) against the lanes' keys, minus the queries' thresholds; f(s0, s1)
+    // unless no key of the wave is seen by the tile.  Pairs outside the mask or the sequence are -inf.
     auto for_tile = [&](int kt, const unsigned char* kt_lds, auto&& f) {
       if (p.causal && kt * kBN + kBN - 1 < wave_row0) return;  // every query of the tile lies before the wave's keys
       const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN < wave_row0 + 31);
