@@ -266,21 +266,6 @@ __device__ __forceinline__ int bwd_seq_len(const AttnBwdParams& p, int b) {
 }
 
 
-// Hardware block ids are dealt round-robin to the 8 XCDs (each with its own L2).  Blocks are renumbered so
-// that every XCD works through whole K/V heads, one after the other, and the K/V heads themselves are dealt
-// round-robin to the XCDs, which keeps right-padded batches balanced.  Returns false for the padding blocks
-// of the grid; `inner` = blocks per K/V head, `unit` / `in_unit` = K/V head index and block index inside it.
-__device__ __forceinline__ bool bwd_block_map(int units, int inner, int& unit, int& in_unit) {
-  const long long total = (long long)units * inner;
-  const long long per_xcd = (total + 7) / 8;
-  const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return false;
-  unit = (int)(logical / inner);
-  in_unit = (int)(logical % inner);
-  if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
-  return true;
-}
-
 // ---------------------------------------------------------------------------------------------------------
 // dQ kernel: one block per (K/V head, query head in its group, row block of 128 queries)
 // ---------------------------------------------------------------------------------------------------------
@@ -306,11 +291,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T
   const int N = p.N;
   const int n_blk = (N + kBwdRows - 1) / kBwdRows;
   const int group = p.Hq / p.Hkv;
-  int bkv, in_unit;
-  if (!bwd_block_map(p.B * p.Hkv, n_blk * group, bkv, in_unit)) return;
-  const int mblk = n_blk - 1 - in_unit / group;  // the longest causal rows first; a group's heads side by side
+  int bkv, mi, hg;
+  if (!xcd_block_map(p.B * p.Hkv, n_blk, group, p.causal != 0, bkv, mi, hg)) return;
+  const int mblk = n_blk - 1 - mi;  // the longest causal rows first; a group's heads side by side
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
-  const int h = kvh * group + in_unit % group;
+  const int h = kvh * group + hg;
   const int bh = b * p.Hq + h;
   // behind the sparse-support dQ kernel: only the row blocks it flagged (all of them when it stepped aside)
   if (p.block_flags && p.queue[kCtrlAllDense] == 0u && (p.queue[kCtrlFlagged] == 0u || p.block_flags[(size_t)bh * n_blk + mblk] == 0)) return;
@@ -533,7 +518,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
   const int N = p.N;
   int bkv, nblk;  // early key blocks have the most causal work and come first
-  if (!bwd_block_map(p.B * p.Hkv, (N + kBwdRows - 1) / kBwdRows, bkv, nblk)) return;
+  int member_unused;
+  if (!xcd_block_map(p.B * p.Hkv, (N + kBwdRows - 1) / kBwdRows, 1, p.causal != 0, bkv, nblk, member_unused)) return;
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int group = p.Hq / p.Hkv;
   // behind the sparse-support dK/dV kernel: only the key blocks it flagged (all of them when it stepped aside)

@@ -70,6 +70,24 @@ template <> __device__ __forceinline__ f32x16 mfma_16bit<f16_t>(u32x4 a, u32x4 b
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
 }
 
+// Sum of four 16-bit values of every lane on the matrix pipe: a 4x4x4 product in 16 blocks of four lanes with A = 1
+// gives each lane, in every register of its accumulator, c + (the sum of its own four B values).  Two passes
+// against the four vector additions it replaces, on a pipe that the vector-bound walks leave idle.
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ f32x4_t lane_sum4(u32x2_t b, f32x4_t c);
+template <> __device__ __forceinline__ f32x4_t lane_sum4<bf16_t>(u32x2_t b, f32x4_t c) {
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  const u32x2_t ones = {0x3f803f80u, 0x3f803f80u};
+  return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, ones), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ f32x4_t lane_sum4<f16_t>(u32x2_t b, f32x4_t c) {
+  typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+  const u32x2_t ones = {0x3c003c00u, 0x3c003c00u};
+  return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h16x4, ones), __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ f32x4_t lane_sum4<float>(u32x2_t, f32x4_t c) { return c; }
+
 // 16-byte global -> LDS copy per lane: lane i of the wave writes LDS bytes [16 i, 16 i + 16) after the
 // wave-uniform base `lds`, from its own global address.
 __device__ __forceinline__ void dma16(const void* gsrc, void* lds) {
@@ -206,25 +224,11 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
   const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
 
-  // ---- XCD-aware block -> (batch, kv head, row block, head in group) mapping -------------------------
-  // Hardware block ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical
-  // ids so the row blocks and grouped heads that share one K/V head hit the same L2.  Inside a K/V head
-  // the longest (last) row blocks of a causal problem go first.
+  // ---- block -> (batch, kv head, row block, head in group): xcd_block_map; causal: longest row blocks first ----
   const int n_mblk = (p.N + BM - 1) / BM;
   const int group = p.Hq / p.Hkv;
-  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
-  const long long per_xcd = (total + 7) / 8;
-  const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return;
-  const int hg = (int)(logical % group);
-  const int mi = (int)((logical / group) % n_mblk);
-  // K/V heads are dealt to the XCDs round-robin rather than in contiguous runs: with right-padded
-  // batches a contiguous run is one batch item, and the XCD that drew the longest sequence would finish last
-  int bkv = (int)(logical / ((long long)group * n_mblk));
-  {
-    const int units = p.B * p.Hkv;
-    if (units % 8 == 0) bkv = (bkv % (units / 8)) * 8 + bkv / (units / 8);
-  }
+  int bkv, mi, hg;
+  if (!xcd_block_map(p.B * p.Hkv, n_mblk, group, p.causal != 0, bkv, mi, hg)) return;
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int h = kvh * group + hg;
   const int mblk = n_mblk - 1 - mi;
@@ -716,134 +720,141 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
     // through a carry-save adder tree (3-input xor / majority, 1 instruction per score) into bit planes:
     // plane k holds bit k of every counter, so a lane keeps 2 x 15 counters of kPlanes bits in kPlanes
     // registers.  Moving the window is one packed shift per plane.
-    constexpr int W = kAttnBins + 1;
-    constexpr int kNoOrigin = -(1 << 29);
-    constexpr int kPlanes = 20;     // a lane meets every other key of its row: up to 2^19 with the 1M-key mask
-    constexpr int kRipple = 9;      // planes below this one take the tile's carry unconditionally
-    constexpr int kTopLo = W, kTopHi = 15;      // bit positions the bin of the maximum may occupy
-    constexpr uint32_t kBinBits = 0xfffefffeu;  // everything but the below-window bit of each half
-    const float c8 = (float)kAttnBins * qs;
-    const float c8n = c8 * (1.f / 65535.f);  // the conversion maps [0, 1] to [0, 65535] and rounds to nearest
-    uint32_t pl[kPlanes];
+    // A counter takes at most 16 entries per key tile (one per word and half), so 12 planes serve walks of up to 255
+    // tiles and 20 planes the longest ones (2^19 entries with the 1M-key mask); the short form keeps 8 registers
+    // fewer alive, ripples its three upper planes without a test and reads out 12 planes instead of 20.
+    auto hist_walk = [&](auto planes_c) {
+      constexpr int kPlanes = decltype(planes_c)::value;
+      constexpr int W = kAttnBins + 1;
+      constexpr int kNoOrigin = -(1 << 29);
+      constexpr int kRipple = 9;      // planes below this one take the tile's carry unconditionally
+      constexpr int kTopLo = W, kTopHi = 15;      // bit positions the bin of the maximum may occupy
+      constexpr uint32_t kBinBits = 0xfffefffeu;  // everything but the below-window bit of each half
+      const float c8 = (float)kAttnBins * qs;
+      const float c8n = c8 * (1.f / 65535.f);  // the conversion maps [0, 1] to [0, 65535] and rounds to nearest
+      uint32_t pl[kPlanes];
 #pragma unroll
-    for (int k = 0; k < kPlanes; ++k) pl[k] = 0u;
-    int g0 = kNoOrigin;
-    // window coordinate y = s c8 - g0 + 1: [0, 1) below the window, [i, i + 1) at bit position i; the
-    // conversion rounds, hence the half
-    float offn = (0.5f - (float)g0) * (1.f / 65535.f);
-    // moves the window up by sh bins (per lane, sh >= 0)
-    auto shift_planes = [&](int sh) {
-      const uint32_t s1 = (uint32_t)(sh < 15 ? sh : 15);
-      const uint32_t s2 = s1 | (s1 << 16);
+      for (int k = 0; k < kPlanes; ++k) pl[k] = 0u;
+      int g0 = kNoOrigin;
+      // window coordinate y = s c8 - g0 + 1: [0, 1) below the window, [i, i + 1) at bit position i; the
+      // conversion rounds, hence the half
+      float offn = (0.5f - (float)g0) * (1.f / 65535.f);
+      // moves the window up by sh bins (per lane, sh >= 0)
+      auto shift_planes = [&](int sh) {
+        const uint32_t s1 = (uint32_t)(sh < 15 ? sh : 15);
+        const uint32_t s2 = s1 | (s1 << 16);
 #pragma unroll
-      for (int k = 0; k < kPlanes; ++k) pl[k] = pk_shr16(pl[k], s2);
-    };
-    tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
-      bool any0 = false, any1 = false;
-      for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
-        float tm0 = s0[0], tm1 = s1[0];
+        for (int k = 0; k < kPlanes; ++k) pl[k] = pk_shr16(pl[k], s2);
+      };
+      tile_loop(nullptr, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
+        bool any0 = false, any1 = false;
+        for_tile(kt, kt_lds, 0.f, [&](const f32x16& s0, const f32x16& s1) {
+          float tm0 = s0[0], tm1 = s1[0];
 #pragma unroll
-        for (int i = 1; i < 16; ++i) {
-          tm0 = fmaxf(tm0, s0[i]);
-          tm1 = fmaxf(tm1, s1[i]);
-        }
-        m_raw = fmaxf(m_raw, fmaxf(tm0, tm1));
-        {
-          // a block matters to the later walks when one of its entries lies within 1 (in z) of the running
-          // maximum; the margin covers the rounding of the difference
-          const float keep = m_raw - inv_qs * 1.0001f - 1e-6f * fabsf(m_raw);
-          any0 = tm0 > keep;
-          any1 = tm1 > keep;
-        }
-        // bin of the maximum; the entries use the same scale, so none lands more than a rounding error above it
-        const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : g0 + kTopLo - 1;
-        int p_top = g_top - g0 + 1;
-        if (__builtin_amdgcn_ballot_w64(p_top > kTopHi) != 0ull) {
-          const int sh = p_top > kTopHi ? p_top - kTopLo : 0;
-          shift_planes(sh);
-          g0 += sh;
-          p_top -= sh;
-          offn = (0.5f - (float)g0) * (1.f / 65535.f);
-        }
-        uint32_t w[16];
+          for (int i = 1; i < 16; ++i) {
+            tm0 = fmaxf(tm0, s0[i]);
+            tm1 = fmaxf(tm1, s1[i]);
+          }
+          m_raw = fmaxf(m_raw, fmaxf(tm0, tm1));
+          {
+            // a block matters to the later walks when one of its entries lies within 1 (in z) of the running
+            // maximum; the margin covers the rounding of the difference
+            const float keep = m_raw - inv_qs * 1.0001f - 1e-6f * fabsf(m_raw);
+            any0 = tm0 > keep;
+            any1 = tm1 > keep;
+          }
+          // bin of the maximum; the entries use the same scale, so none lands more than a rounding error above it
+          const int g_top = m_raw > -INFINITY ? (int)floorf(m_raw * c8) : g0 + kTopLo - 1;
+          int p_top = g_top - g0 + 1;
+          if (__builtin_amdgcn_ballot_w64(p_top > kTopHi) != 0ull) {
+            const int sh = p_top > kTopHi ? p_top - kTopLo : 0;
+            shift_planes(sh);
+            g0 += sh;
+            p_top -= sh;
+            offn = (0.5f - (float)g0) * (1.f / 65535.f);
+          }
+          uint32_t w[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const float sa = j < 8 ? s0[(2 * j) & 15] : s1[(2 * j) & 15];
-          const float sb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
-          w[j] = pk_shl16(0x00010001u, __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_u16(fmaf(sa, c8n, offn), fmaf(sb, c8n, offn))));
-        }
-        // adder tree: 16 words + plane 0 -> plane 0 and 8 carries, those + plane 1 -> plane 1 and 4 carries, ...
-        uint32_t c2[8], c4[4], c8w[2], c16;
-        uint32_t acc = pl[0];
+          for (int j = 0; j < 16; ++j) {
+            const float sa = j < 8 ? s0[(2 * j) & 15] : s1[(2 * j) & 15];
+            const float sb = j < 8 ? s0[(2 * j + 1) & 15] : s1[(2 * j + 1) & 15];
+            w[j] = pk_shl16(0x00010001u, __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_u16(fmaf(sa, c8n, offn), fmaf(sb, c8n, offn))));
+          }
+          // adder tree: 16 words + plane 0 -> plane 0 and 8 carries, those + plane 1 -> plane 1 and 4 carries, ...
+          uint32_t c2[8], c4[4], c8w[2], c16;
+          uint32_t acc = pl[0];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) full_add(acc, w[2 * j], w[2 * j + 1], acc, c2[j]);
-        pl[0] = acc;
-        acc = pl[1];
+          for (int j = 0; j < 8; ++j) full_add(acc, w[2 * j], w[2 * j + 1], acc, c2[j]);
+          pl[0] = acc;
+          acc = pl[1];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) full_add(acc, c2[2 * j], c2[2 * j + 1], acc, c4[j]);
-        pl[1] = acc;
-        acc = pl[2];
+          for (int j = 0; j < 4; ++j) full_add(acc, c2[2 * j], c2[2 * j + 1], acc, c4[j]);
+          pl[1] = acc;
+          acc = pl[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) full_add(acc, c4[2 * j], c4[2 * j + 1], acc, c8w[j]);
-        pl[2] = acc;
-        acc = pl[3];
-        full_add(acc, c8w[0], c8w[1], acc, c16);
-        pl[3] = acc;
-        // the carry out of the tree ripples through the next planes; a carry into plane kRipple is rare enough
-        // for a branch.  The below-window bit would carry on every tile and is dropped.
-        uint32_t carry = c16 & kBinBits;
+          for (int j = 0; j < 2; ++j) full_add(acc, c4[2 * j], c4[2 * j + 1], acc, c8w[j]);
+          pl[2] = acc;
+          acc = pl[3];
+          full_add(acc, c8w[0], c8w[1], acc, c16);
+          pl[3] = acc;
+          // the carry out of the tree ripples through the next planes; a carry into plane kRipple is rare enough
+          // for a branch.  The below-window bit would carry on every tile and is dropped.
+          uint32_t carry = c16 & kBinBits;
 #pragma unroll
-        for (int k = 4; k < kRipple; ++k) {
-          const uint32_t t = pl[k] & carry;
-          pl[k] ^= carry;
-          carry = t;
-        }
-        if (__builtin_amdgcn_ballot_w64(carry != 0u) != 0ull) {
-#pragma unroll
-          for (int k = kRipple; k < kPlanes; ++k) {
+          for (int k = 4; k < kRipple; ++k) {
             const uint32_t t = pl[k] & carry;
             pl[k] ^= carry;
             carry = t;
           }
+          if (kPlanes - kRipple <= 3 || __builtin_amdgcn_ballot_w64(carry != 0u) != 0ull) {
+#pragma unroll
+            for (int k = kRipple; k < kPlanes; ++k) {
+              const uint32_t t = pl[k] & carry;
+              pl[k] ^= carry;
+              carry = t;
+            }
+          }
+        });
+        if constexpr (kFine) {
+          const uint32_t nb = (__builtin_amdgcn_ballot_w64(any0) != 0ull ? 1u : 0u) | (__builtin_amdgcn_ballot_w64(any1) != 0ull ? 2u : 0u);
+          if (nb && lane == 0) mark_blocks(mask_new, fine_new, kt, nb);
+        } else {
+          if (__builtin_amdgcn_ballot_w64(any0 || any1) != 0ull && lane == 0) mark_tile(mask_new, kt);
         }
       });
-      if constexpr (kFine) {
-        const uint32_t nb = (__builtin_amdgcn_ballot_w64(any0) != 0ull ? 1u : 0u) | (__builtin_amdgcn_ballot_w64(any1) != 0ull ? 2u : 0u);
-        if (nb && lane == 0) mark_blocks(mask_new, fine_new, kt, nb);
-      } else {
-        if (__builtin_amdgcn_ballot_w64(any0 || any1) != 0ull && lane == 0) mark_tile(mask_new, kt);
+      // the two lanes of a row bring their windows to the row's nine bins, bin g_top - 8 at bit position 1; then
+      // the counters are read out of the planes (both halves of a word belong to the lane's row) and added up
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
+      const int g0_row = (m_raw > -INFINITY ? (int)floorf(m_raw * c8) : kNoOrigin + kAttnBins) - kAttnBins;
+      shift_planes(g0_row - g0);  // >= 0: a lane's window starts at or below its own maximum's ninth bin
+      float cnt[W];
+#pragma unroll
+      for (int bin = 0; bin < W; ++bin) {
+        uint32_t c = 0u;
+#pragma unroll
+        for (int k = 0; k < kPlanes; ++k) {
+          uint32_t bits = ((pl[k] >> (bin + 1)) & 1u) + ((pl[k] >> (bin + 17)) & 1u);
+          // an entry a rounding error above the top bin counts as sitting in it
+          if (bin == W - 1) bits += ((pl[k] >> (bin + 2)) & 1u) + ((pl[k] >> (bin + 18)) & 1u);
+          c += bits << k;
+        }
+        cnt[bin] = (float)c;
       }
-    });
-    // the two lanes of a row bring their windows to the row's nine bins, bin g_top - 8 at bit position 1; then
-    // the counters are read out of the planes (both halves of a word belong to the lane's row) and added up
-    m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, 64));
-    const int g0_row = (m_raw > -INFINITY ? (int)floorf(m_raw * c8) : kNoOrigin + kAttnBins) - kAttnBins;
-    shift_planes(g0_row - g0);  // >= 0: a lane's window starts at or below its own maximum's ninth bin
-    float cnt[W];
 #pragma unroll
-    for (int bin = 0; bin < W; ++bin) {
-      uint32_t c = 0u;
+      for (int k = 0; k < W; ++k) cnt[k] += __shfl_xor(cnt[k], 32, 64);
+      // Every entry counts as sitting on the lower edge of its bin, which gives a lower bound of tau that is
+      // less than one bin width off (the entries left out lie below max - 1).
+      const float t_shift = (float)g0_row * kBinW;
+      hist_lo = (AM == ATT_15) ? hist_bracket_alpha15<W>(cnt, t_shift, kBinW) : hist_bracket_alpha2<W>(cnt, t_shift, kBinW);
+      {
+        float n_cand = 0.f;  // the entries of the bins that reach above the bound
 #pragma unroll
-      for (int k = 0; k < kPlanes; ++k) {
-        uint32_t bits = ((pl[k] >> (bin + 1)) & 1u) + ((pl[k] >> (bin + 17)) & 1u);
-        // an entry a rounding error above the top bin counts as sitting in it
-        if (bin == W - 1) bits += ((pl[k] >> (bin + 2)) & 1u) + ((pl[k] >> (bin + 18)) & 1u);
-        c += bits << k;
+        for (int k = 0; k < W; ++k) n_cand += (t_shift + (float)(k + 1) * kBinW > hist_lo) ? cnt[k] : 0.f;
+        cand_est = wave_sum(lh == 0 && qi < L ? n_cand : 0.f);
       }
-      cnt[bin] = (float)c;
-    }
-#pragma unroll
-    for (int k = 0; k < W; ++k) cnt[k] += __shfl_xor(cnt[k], 32, 64);
-    // Every entry counts as sitting on the lower edge of its bin, which gives a lower bound of tau that is
-    // less than one bin width off (the entries left out lie below max - 1).
-    const float t_shift = (float)g0_row * kBinW;
-    hist_lo = (AM == ATT_15) ? hist_bracket_alpha15<W>(cnt, t_shift, kBinW) : hist_bracket_alpha2<W>(cnt, t_shift, kBinW);
-    {
-      float n_cand = 0.f;  // the entries of the bins that reach above the bound
-#pragma unroll
-      for (int k = 0; k < W; ++k) n_cand += (t_shift + (float)(k + 1) * kBinW > hist_lo) ? cnt[k] : 0.f;
-      cand_est = wave_sum(lh == 0 && qi < L ? n_cand : 0.f);
-    }
+    };
+    if (nt <= 255) hist_walk(std::integral_constant<int, 12>{});
+    else hist_walk(std::integral_constant<int, 20>{});
     mask_cur = mask_new;
     mask_new = mask_b;
     fine_new = fine_of(mask_new);
@@ -929,6 +940,10 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
       bool build = kWithLists && !list_mode && may_build && want_lists;  // uniform over the wave
       bool lane_full = false;
       const bool collecting = build;
+      // The block maxima serve the tile mask of the next walk (and the lists).  When the histogram has counted, over
+      // the wave's 32 rows, several candidates per key tile, no tile will drop out for this wave and the maxima are
+      // not worth their instructions (uniform over the wave).
+      const bool track = build || !(with_hist && cand_est > 4.f * (float)nt);
       // the lane's candidates of a block join its list; the wave stops collecting once a lane is out of room
       auto append_block = [&](const f32x16& sc, int key0) {  // key0: the lane's first key of the block
 #pragma unroll
@@ -975,33 +990,42 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
           // v_pk_fma_f16 / v_pk_add_f16 and not the two-term dot product with fp32 accumulation: on this part a
           // wave's v_dot2 instructions and another wave's MFMAs exclude each other completely, while the other
           // vector instructions give up less than half of an MFMA's duration.
-          const h2_t ninf2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
-          h2_t dm2[2] = {ninf2, ninf2};
-          const h2_t zero2 = {(_Float16)0.f, (_Float16)0.f};
-          h2_t sq2 = zero2, su2 = zero2;
-          for_tile_sel(kt, kt_lds, init, bits, [&](const f32x16& sc, int kb) {
-            n_seen += 16;
+          auto packed_tile = [&](auto track_c) {
+            constexpr bool kTrack = decltype(track_c)::value;
+            const h2_t ninf2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+            const h2_t pinf2 = {(_Float16)INFINITY, (_Float16)INFINITY};
+            // (a wave that does not track the block maxima marks every tile it visits)
+            h2_t dm2[2] = {kTrack ? ninf2 : pinf2, kTrack ? ninf2 : pinf2};
+            const h2_t zero2 = {(_Float16)0.f, (_Float16)0.f};
+            h2_t sq2 = zero2, su2 = zero2;
+            for_tile_sel(kt, kt_lds, init, bits, [&](const f32x16& sc, int kb) {
+              n_seen += 16;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float ra = sc[2 * j];
-              const float rb = sc[2 * j + 1];
-              const h2_t h = pkrtz(ra, rb);
-              dm2[kb] = __builtin_elementwise_max(dm2[kb], h);
-              cnt_neg += __builtin_popcount(__builtin_bit_cast(uint32_t, h) & 0x80008000u);
-              const h2_t u = __builtin_elementwise_max(h, zero2);
-              if constexpr (AM == ATT_15) sq2 = __builtin_elementwise_fma(u, u, sq2);
-              su2 = su2 + u;
+              for (int j = 0; j < 8; ++j) {
+                const float ra = sc[2 * j];
+                const float rb = sc[2 * j + 1];
+                const h2_t h = pkrtz(ra, rb);
+                if constexpr (kTrack) dm2[kb] = __builtin_elementwise_max(dm2[kb], h);
+                // population count with the running total as its addend: one instruction
+                asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(cnt_neg) : "v"(__builtin_bit_cast(uint32_t, h) & 0x80008000u));
+                const h2_t u = __builtin_elementwise_max(h, zero2);
+                if constexpr (AM == ATT_15) sq2 = __builtin_elementwise_fma(u, u, sq2);
+                su2 = su2 + u;
+              }
+              if constexpr (kTrack)
+                if (build && __builtin_amdgcn_ballot_w64(live_row && fmaxf((float)dm2[kb][0], (float)dm2[kb][1]) > dl) != 0ull) append_block(sc, kt * kBN + kb * 32 + 4 * lh);
+            });
+            if constexpr (AM == ATT_15) {
+              a0 += (float)sq2[0] + (float)sq2[1];
+              a1 += (float)su2[0] + (float)su2[1];
+            } else {
+              a0 += (float)su2[0] + (float)su2[1];
             }
-            if (build && __builtin_amdgcn_ballot_w64(live_row && fmaxf((float)dm2[kb][0], (float)dm2[kb][1]) > dl) != 0ull) append_block(sc, kt * kBN + kb * 32 + 4 * lh);
-          });
-          if constexpr (AM == ATT_15) {
-            a0 += (float)sq2[0] + (float)sq2[1];
-            a1 += (float)su2[0] + (float)su2[1];
-          } else {
-            a0 += (float)su2[0] + (float)su2[1];
-          }
-          dmax0 = fmaxf((float)dm2[0][0], (float)dm2[0][1]);
-          dmax1 = fmaxf((float)dm2[1][0], (float)dm2[1][1]);
+            dmax0 = fmaxf((float)dm2[0][0], (float)dm2[0][1]);
+            dmax1 = fmaxf((float)dm2[1][0], (float)dm2[1][1]);
+          };
+          if (track) packed_tile(std::true_type{});
+          else packed_tile(std::false_type{});
         } else {
           for_tile_sel(kt, kt_lds, init, bits, [&](const f32x16& sc, int kb) {
             float dm = -INFINITY;
@@ -1073,6 +1097,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float psum = 0.f;
+  f32x4_t psum4 = {0.f, 0.f, 0.f, 0.f};  // 16-bit walks: every register holds the lane's sum
   unsigned active16 = 0;  // 16x16 score tiles with a non-zero probability (wave-uniform count)
   // With the lists in place (and no tile statistics asked for) there is nothing to walk: a lane turns its
   // listed scores into probabilities and adds up the V rows of their keys, read from the row-major V.
@@ -1158,15 +1183,31 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
       };
       for_tile_blocks(kt, kt_lds, init, bits, [&](const f32x16& acc, int kb) {
         float pv[16];
-        float hsum[2] = {0.f, 0.f};  // over the lane's keys of each 16-key half of the block
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          pv[i] = attn_prob<AM>(acc[i], qs, p.c0);
-          hsum[i >> 3] += pv[i];
+        for (int i = 0; i < 16; ++i) pv[i] = attn_prob<AM>(acc[i], qs, p.c0);
+        // 16-bit types: the probabilities are rounded to the operand format first; their sum is taken from the
+        // rounded values (what the product below really weighs V with) on the matrix pipe, and "is there anything in
+        // this 16-key half" from the or of the packed words.  fp32: plain sums.
+        u32x4 bp[2];
+        bool half_live[2];  // over the lane's keys of each 16-key half of the block
+        if constexpr (k16) {
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            bp[s] = u32x4{pack2<T>(pv[8 * s], pv[8 * s + 1]), pack2<T>(pv[8 * s + 2], pv[8 * s + 3]),
+                          pack2<T>(pv[8 * s + 4], pv[8 * s + 5]), pack2<T>(pv[8 * s + 6], pv[8 * s + 7])};
+            half_live[s] = ((bp[s][0] | bp[s][1]) | (bp[s][2] | bp[s][3])) != 0u;
+            psum4 = lane_sum4<T>(u32x2_t{bp[s][0], bp[s][1]}, psum4);
+            psum4 = lane_sum4<T>(u32x2_t{bp[s][2], bp[s][3]}, psum4);
+          }
+        } else {
+          float hsum[2] = {0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < 16; ++i) hsum[i >> 3] += pv[i];
+          psum += hsum[0] + hsum[1];
+          half_live[0] = hsum[0] > 0.f;
+          half_live[1] = hsum[1] > 0.f;
         }
-        const float bsum = hsum[0] + hsum[1];
-        psum += bsum;
-        tile_active |= bsum > 0.f;
+        tile_active |= half_live[0] || half_live[1];
         if (p.tile_counts) {
           // lanes 0-15 / 32-47 hold query rows 0-15, lanes 16-31 / 48-63 rows 16-31; registers 0-7 hold
           // keys 0-15 of the block, registers 8-15 keys 16-31.
@@ -1190,15 +1231,13 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
           for (int s = 0; s < 2; ++s) {
             // a 16-key half in which no row of the wave has a non-zero probability adds nothing: with a
             // support of a few keys per row that is a large share of the halves
-            if (__builtin_amdgcn_ballot_w64(hsum[s] > 0.f) == 0ull) continue;
-            u32x4 bp = {pack2<T>(pv[8 * s], pv[8 * s + 1]), pack2<T>(pv[8 * s + 2], pv[8 * s + 3]),
-                        pack2<T>(pv[8 * s + 4], pv[8 * s + 5]), pack2<T>(pv[8 * s + 6], pv[8 * s + 7])};
+            if (__builtin_amdgcn_ballot_w64(half_live[s]) == 0ull) continue;
 #pragma unroll
             for (int db = 0; db < G::kDB; ++db) {
               const int drow = db * 32 + lq;
               u32x4 a = {0u, 0u, 0u, 0u};
               if (D >= 32 || drow < D) a = lds_read16(va ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
-              o[db] = mfma_16bit<T>(a, bp, o[db]);
+              o[db] = mfma_16bit<T>(a, bp[s], o[db]);
             }
           }
         } else {
@@ -1223,6 +1262,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
         mark_tile(mask_out0 + half * p.mask_words, kt);
     });
   }
+  psum += psum4[0];
   psum += __shfl_xor(psum, 32, 64);
   const float inv = psum > 0.f ? 1.f / psum : 0.f;
 

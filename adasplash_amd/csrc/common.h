@@ -103,6 +103,48 @@ __device__ __forceinline__ int wave_sum_i(int v) {
   return v;
 }
 
+// ---- block numbering of the dense attention kernels -------------------------------------------------------
+// Hardware block ids are dealt round-robin to the 8 XCDs (one L2 each): XCD x runs the blocks x, x + 8, ... in
+// that order, a new one whenever a slot of its 32 CUs falls free.  The K/V heads (`units`) are dealt round-robin
+// to the XCDs -- with right-padded batches a contiguous run of heads is one batch item, and the XCD that drew
+// the longest sequence would finish last -- and an XCD works through its heads in sets.  A set is one head when
+// the blocks cost the same (`balance` false) or a head alone has several blocks per slot; its K and V then stay
+// in that L2.  When the blocks of a head differ in cost (causal: block index 0 is the longest) and a head has
+// few of them, a set takes as many heads as give about two blocks per slot and runs them longest block first
+// over all its heads: started in that order, the short blocks fill the slots the long ones leave, where head
+// after head the last head's longest block would start when the others are almost through.
+// `blocks` = blocks per (head, member of its group), `group` = query heads per K/V head; returns false for the
+// padding blocks of the grid, else the K/V head, the block index and the member.
+__device__ __forceinline__ bool xcd_block_map(int units, int blocks, int group, bool balance, int& unit, int& blk, int& member) {
+  const int inner = blocks * group;
+  const int x = (int)(blockIdx.x & 7);
+  const long long seq = (long long)(blockIdx.x >> 3);
+  if (units % 8 != 0) {
+    const long long total = (long long)units * inner;
+    const long long per_xcd = (total + 7) / 8;
+    const long long logical = x * per_xcd + seq;
+    if (seq >= per_xcd || logical >= total) return false;
+    unit = (int)(logical / inner);
+    blk = (int)(logical % inner) / group;
+    member = (int)(logical % inner) % group;
+    return true;
+  }
+  const int upx = units / 8;  // heads of this XCD
+  if (seq >= (long long)upx * inner) return false;
+  constexpr int kSetBlocks = 256;  // two blocks for each of 32 CUs x 4 resident blocks
+  int g = balance ? (kSetBlocks + inner - 1) / inner : 1;
+  g = g < upx ? g : upx;
+  const int set = (int)(seq / ((long long)g * inner));
+  const int s = (int)(seq - (long long)set * g * inner);
+  const int gsize = (upx - set * g) < g ? (upx - set * g) : g;
+  const int span = gsize * group;
+  blk = s / span;
+  const int r = s % span;
+  unit = (set * g + r / group) * 8 + x;
+  member = r % group;
+  return true;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
