@@ -327,8 +327,10 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
                        (const uint32_t*)p.queue);
   }
   // The list-carrying instance serves two and more solver steps, and a single step without the histogram (the
-  // block-mask variant's, made for sparse supports); the other one no step, or one behind the histogram.
-  const bool multi = niter >= 2 || (niter == 1 && !use_hist);
+  // block-mask variant's, made for sparse supports); the other one no step, or one behind the histogram -- and
+  // whatever the sparse-support kernel leaves over: those row blocks did not fit its lists, which are longer than
+  // this kernel's, so they are walked step by step, and the walk-only instance does that with fewer registers.
+  const bool multi = (niter >= 2 || (niter == 1 && !use_hist)) && p.queue == nullptr;
   int rc = kFwdTable[dtype][head_dim_slot(D)][multi ? 1 : 0](p, am, s);
   if (rc != 0) return ADSP_ERR_LAUNCH;
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;

@@ -141,12 +141,12 @@ def test_bench_shapes_downscaled_bf16(niter):
     q = (torch.randn(1, 4, 1024, 64) / 8).to(torch.bfloat16)
     k, v = (torch.randn(1, 4, 1024, 64).to(torch.bfloat16) for _ in range(2))
     tol = 2e-2 if niter >= 1 else 0.5  # niter = 0: no refinement, tau is the midpoint of the 1/8-wide histogram bracket
-    assert max_err(run_v2(q, k, v, niter=niter), exact.dense_entmax_attention(q, k, v, 1.5, True)) < tol
+    assert max_err(run_v2(q, k, v, niter=niter), exact.dense_entmax_attention(q, k, v, 1.5, True), report=niter >= 1) < tol
     q = torch.randn(2, 8, 1024, 128).to(torch.bfloat16)
     k, v = (torch.randn(2, 2, 1024, 128).to(torch.bfloat16) for _ in range(2))
     varlen = torch.tensor([1024, 300], dtype=torch.int32)
     out = run_v2(q, k, v, niter=niter, varlen=varlen)
-    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen)) < tol
+    assert max_err(out, exact.dense_entmax_attention(q, k, v, 1.5, True, varlen), report=niter >= 1) < tol
 
 
 def test_thresholds_support_and_block_mask():
