@@ -207,9 +207,9 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
   if (dense_rows >= 3) ctrl[64 + 2 * u] = 1u << 20;  // (the sparse kernel counts the marked heads itself)
 }
 
-// Workspace of the forward for the 16-bit types: the key-major copy of V, then -- for the head dims the
-// sparse-support kernel serves -- its work counters, its per-row-block flags, its candidate streams and the e4m3 copy
-// of K that its first walk reads.
+// Workspace of the forward for the 16-bit types, for the head dims the sparse-support kernel serves: its work
+// counters, its per-row-block flags, its candidate streams and the e4m3 copy of K that its first walk reads.  (The
+// dense kernel needs none: it reads V row-major and transposes in the LDS read.)
 constexpr int kSparseMaxSlots = 1024;                       // workgroups of the persistent kernel
 constexpr size_t kSparseSlotBytes = (size_t)4 * 1616 * 8;   // four waves x 1616 candidates x (score, key)
 struct FwdWorkspace {
@@ -220,8 +220,8 @@ static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
   FwdWorkspace w = {};
   if (dtype == ADSP_F32) return w;
-  w.vt_bytes = (size_t)B * Hkv * D * npad_of(N) * 2;
-  w.total = w.vt_bytes;
+  w.vt_bytes = 0;
+  w.total = 0;
   if ((D == 64 || D == 128) && N <= 65536) {  // (the candidate lists hold 16-bit key indices)
     const long long items = (long long)B * Hq * mblocks_of(N);
     long long slots = (items + 7) / 8 * 8;
@@ -296,9 +296,8 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
     const FwdWorkspace w = fwd_workspace(B, Hq, Hkv, N, D, dtype);
-    if (!workspace || workspace_bytes < w.total || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
+    if (w.total && (!workspace || workspace_bytes < w.total || ((uintptr_t)workspace & 15) != 0)) return ADSP_ERR_WORKSPACE;
     unsigned char* ws = (unsigned char*)workspace;
-    p.vt = workspace;
     // Sparse-support kernel first (alpha 1.5 / 2, either entry point, no tile statistics asked for): it serves the
     // row blocks whose supports are short and flags the others for the kernel below.
     const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && !tile_counts &&
@@ -321,10 +320,6 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
                                   : (D == 64 ? launch_attn_sparse_f16_d64(p, am, w.slots, s) : launch_attn_sparse_f16_d128(p, am, w.slots, s));
       if (rc != 0) return ADSP_ERR_LAUNCH;
     }
-    // the key-major copy of V serves the dense kernel only
-    hipLaunchKernelGGL(vt_layout_kernel, dim3(vt_layout_blocks(p.Npad, D), (unsigned)(B * Hkv)), dim3(256), 0, s,
-                       (const uint16_t*)v, (uint16_t*)workspace, N, p.Npad, D, varlen, varlen_bits, Hkv,
-                       (const uint32_t*)p.queue);
   }
   // The list-carrying instance serves two and more solver steps, and a single step without the histogram (the
   // block-mask variant's, made for sparse supports); the other one no step, or one behind the histogram -- and

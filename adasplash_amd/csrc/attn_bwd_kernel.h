@@ -45,7 +45,8 @@ template <int AM> __device__ __forceinline__ void bwd_prob(float r, float c0, fl
 template <typename T, int D> struct BwdTiles {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
-  using VS = Swz<G::kVRow>;
+  static constexpr int kTRow = G::k16 ? kBN * 2 : D * 4;  // 16-bit: a row of a transposed tile [D][64 keys]; fp32: of a [64][D] tile
+  using VS = Swz<kTRow>;
   static constexpr bool k16 = G::k16;
   static constexpr int kTile = G::kKTile;  // bytes of a [64][D] tile, in either orientation
   static constexpr int kNW = kBwdRows / 32;
@@ -96,7 +97,7 @@ template <typename T, int D> struct BwdTiles {
       if (kLoads % kNW == 0 || j < kLoads) {
         const int P = j * 64 + lane;
         const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
-        dma16s(gtile, (uint32_t)(row * G::kVRow + c * 16), lds + j * 1024);
+        dma16s(gtile, (uint32_t)(row * kTRow + c * 16), lds + j * 1024);
       }
     }
   }
@@ -189,7 +190,7 @@ template <typename T, int D> struct BwdTiles {
       }
     } else if constexpr (k16) {
       // same addressing for the transposed tile: chunk 4 kb + 2 s + lh of row 32 db + lq
-      uint32_t ta = (uint32_t)(uintptr_t)tile + (uint32_t)(lq * G::kVRow + ((lh ^ VS::sw(lq)) << 4));
+      uint32_t ta = (uint32_t)(uintptr_t)tile + (uint32_t)(lq * kTRow + ((lh ^ VS::sw(lq)) << 4));
       asm volatile("" : "+v"(ta));
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
@@ -199,7 +200,7 @@ template <typename T, int D> struct BwdTiles {
         for (int db = 0; db < G::kDB; ++db) {
           const int drow = db * 32 + lq;
           u32x4 a = {0u, 0u, 0u, 0u};
-          if (D >= 32 || drow < D) a = lds_read16(ta ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
+          if (D >= 32 || drow < D) a = lds_read16(ta ^ ((kb * 4 + 2 * s) << 4), db * 32 * kTRow);
           o[db] = mfma_16bit<T>(a, b, o[db]);
         }
       }

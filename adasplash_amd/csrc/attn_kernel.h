@@ -126,6 +126,15 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr, int imm = 0) {
   return *(const __attribute__((address_space(3))) u32x4*)(addr + imm);
 }
 
+// 8-byte transposing LDS read (ds_read_b64_tr_b16): within every group of 16 lanes, lane 4 r + c gives the address of four
+// consecutive 16-bit values, and lane j receives, as its element r, value j % 4 of the four that lane 4 r + j / 4
+// addressed.  With lane 4 r + c pointing at columns 4 c .. 4 c + 3 of row r of a row-major tile, lane j ends up with
+// column j of rows 0 .. 3: an MFMA operand that runs along the rows, from a tile stored along the columns.
+__device__ __forceinline__ u32x2_t lds_read8_tr(uint32_t addr, int imm = 0) {
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + imm)));
+}
+
 // Tile geometry.  A tile row has kC 16-byte chunks; chunk c of row r is stored at chunk position
 // c ^ sw(r), with sw chosen so that 16 consecutive rows reading the same logical chunk touch 16 different
 // 16-byte bank groups.
@@ -142,8 +151,8 @@ template <typename T, int D> struct TileGeo {
   static constexpr int kEB = k16 ? 2 : 4;
   static constexpr int kKRow = D * kEB;                // bytes per key row of the K tile
   static constexpr int kKTile = kBN * kKRow;
-  static constexpr int kVRow = k16 ? kBN * 2 : D * 4;  // 16-bit: V^T tile [D][64 keys]; fp32: V tile [64][D]
-  static constexpr int kVRows = k16 ? D : kBN;
+  static constexpr int kVRow = kKRow;  // the V tile has the K tile's format: [64 keys][D], row-major
+  static constexpr int kVRows = kBN;
   static constexpr int kVTile = kVRows * kVRow;
   static constexpr int kNBuf = (2 * (kKTile + kVTile) <= 144 * 1024) ? 2 : 1;
   // Workgroups of four waves; two to four of them share a CU (registers and LDS permitting), one wave of each
@@ -298,9 +307,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
 
   // ---- tile DMA ---------------------------------------------------------------------------------------
   const unsigned char* kglob = reinterpret_cast<const unsigned char*>(p.k) + kv_base * G::kEB;
-  const unsigned char* vglob =
-      k16 ? reinterpret_cast<const unsigned char*>(p.vt) + ((size_t)(b * p.Hkv + kvh) * D) * p.Npad * 2
-          : reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kEB;
+  const unsigned char* vglob = reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kEB;
 
   // Wave-level load j of a tile fills LDS bytes [1024 j, 1024 j + 1024): chunk position P = 64 j + lane
   // belongs to row P / kC, stored chunk P % kC, i.e. logical chunk (P % kC) ^ sw(row).
@@ -309,34 +316,56 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   // A wave's successive loads of a tile lie NW KB apart and NW * 64 / kC rows further down; when that is a multiple of
   // the swizzle period (16 rows) the lane's offset of load j0 is that of load 0 plus j0 * NW KB, which goes into the
   // scalar base: one offset register per tile kind instead of one per load.
-  constexpr int kKPer = (G::kKLoads + NW - 1) / NW, kVPer = (G::kVLoads + NW - 1) / NW;
+  constexpr int kKPer = (G::kKLoads + NW - 1) / NW;
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
-  constexpr bool kVStep = (NW * 64 / VS::kC) % 16 == 0 && (NW * 64) % VS::kC == 0;
-  constexpr int kKOffs = kKStep ? 1 : kKPer, kVOffs = kVStep ? 1 : kVPer;
-  uint32_t koff[kKOffs], voff[kVOffs];
+  constexpr int kKOffs = kKStep ? 1 : kKPer;
+  uint32_t koff[kKOffs], voff[kKOffs];
+  // The 16-bit V tile has a swizzle of its own, made for the transposing reads of the output product: the four rows
+  // that the 16 lanes of a group address together (keys x .. x + 3, 32 bytes of each) must fall into four different
+  // quarters of the 128 bytes that the banks serve per cycle, i.e. differ in bits 1 and 2 of their chunk position.
+  // Its period (4 rows) divides that of the K tile's, so the scalar-base stepping of the loads holds for both.
+  auto vsw = [](int row) -> int {
+    if constexpr (k16) {
+      constexpr int kC = KS::kC;
+      if constexpr (kC >= 8) return (2 * row) & ((kC >= 16 ? 16 : kC) - 1);
+      else if constexpr (kC == 4) return row & 2;
+      else return 0;
+    } else {
+      return KS::sw(row);
+    }
+  };
 #pragma unroll
   for (int j0 = 0; j0 < kKOffs; ++j0) {
     const int P = (j0 * NW + wave) * 64 + lane;
     const int row = P / KS::kC;
     koff[j0] = (uint32_t)(row * G::kKRow + (((P % KS::kC) ^ KS::sw(row)) << 4));
-  }
-#pragma unroll
-  for (int j0 = 0; j0 < kVOffs; ++j0) {
-    const int P = (j0 * NW + wave) * 64 + lane;
-    const int row = P / VS::kC;
-    voff[j0] = (uint32_t)(row * G::kVRow + (((P % VS::kC) ^ VS::sw(row)) << 4));
+    voff[j0] = (uint32_t)(row * G::kKRow + (((P % KS::kC) ^ vsw(row)) << 4));
   }
   // Swizzled read addresses without a register per fragment (three or four waves per SIMD leave none to spare): chunk c
   // of row r sits at r * row_bytes + ((c ^ sw(r)) << 4), and with c = 2 ks + lh that is
   // (r * row_bytes + ((lh ^ sw(r)) << 4)) ^ (ks << 5) -- one lane constant and one xor with an immediate per
-  // read.  Rows r and r + 32 share sw, so the second key block is an offset.  Same for the V^T tile with
-  // c = 4 kb + 2 s + lh.
+  // read.  Rows r and r + 32 share sw, so the second key block is an offset.
   const uint32_t k_lane = (uint32_t)(lq * G::kKRow + ((lh ^ KS::sw(lq)) << 4));
-  const uint32_t v_lane = (uint32_t)(lq * G::kVRow + ((lh ^ VS::sw(lq)) << 4));
-  auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKOffs], unsigned char* lds, int kt) {
-    // a row-major [64][D] tile out of a row-major tensor (K, or V for fp32); the last tile may stick out
+  // The V operand of the output product (16-bit): out^T = V^T P^T wants, per lane, one output column d and eight keys
+  // of a 16-key half -- in the order the score registers hold them: keys 4 g .. 4 g + 3 and 8 + 4 g .. 8 + 4 g + 3 for the
+  // lane's half g = lane / 32 -- out of the row-major tile.  Two transposing reads bring them: in a group of 16 lanes,
+  // lane 4 r + c points at key (4 g + r [+ 8]) and columns 4 c .. 4 c + 3 of the group's 16 columns (groups 0 / 2: columns
+  // 0 .. 15 of a block of 32, groups 1 / 3: 16 .. 31).  The swizzle of these keys does not depend on the 16-key half, so the
+  // lane's offsets are constants; the block of 32 columns is an xor with an immediate.
+  uint32_t v_lane[2];
+  {
+    const int a = lane & 15, grp = lane >> 4, r = a >> 2, c = a & 3, g = grp >> 1, dl = grp & 1;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const int x = 4 * g + r + 8 * w;
+      v_lane[w] = (uint32_t)(x * G::kVRow + (((2 * dl + (c >> 1)) ^ vsw(x)) << 4) + (c & 1) * 8);
+    }
+    if (D < 32 && dl) v_lane[0] = v_lane[1] = 0u;  // (D = 16: these lanes' columns do not exist; their operand is zeroed)
+  }
+  auto issue_rows = [&](const unsigned char* g, const uint32_t (&off)[kKOffs], unsigned char* lds, int kt, int limit, auto&& sw_of) {
+    // a row-major [64][D] tile out of a row-major tensor (K or V); the last tile may stick out of the rows [0, limit)
     const unsigned char* base = uniform_ptr(g + (size_t)kt * G::kKTile);
-    if ((kt + 1) * kBN <= N) {  // one branch per tile, then straight-line loads
+    if ((kt + 1) * kBN <= limit) {  // one branch per tile, then straight-line loads
 #pragma unroll
       for (int j0 = 0; j0 < kKPer; ++j0) {
         const int j = j0 * NW + wave;
@@ -351,30 +380,18 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
         const int j = j0 * NW + wave;
         if (G::kKLoads % NW == 0 || j < G::kKLoads) {
           const int P = j * 64 + lane;
-          const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
+          const int row = P / KS::kC, c = (P % KS::kC) ^ sw_of(row);
           int gk = kt * kBN + row;
-          gk = gk < N ? gk : N - 1;  // rows past the end are masked later; any valid row will do
+          gk = gk < limit ? gk : limit - 1;  // rows past the end are masked later; any valid row will do
           dma16(g + (size_t)gk * G::kKRow + c * 16, lds + j * 1024);
         }
       }
     }
   };
-  auto issue_k = [&](unsigned char* kb, int kt) { issue_rows(kglob, koff, kb, kt); };
-  auto issue_v = [&](unsigned char* vb, int kt) {
-    if constexpr (k16) {
-      const unsigned char* base = uniform_ptr(vglob + (size_t)kt * G::kVTile);  // the transposed copy is padded to whole tiles
-#pragma unroll
-      for (int j0 = 0; j0 < kVPer; ++j0) {
-        const int j = j0 * NW + wave;
-        if (G::kVLoads % NW == 0 || j < G::kVLoads) {
-          if constexpr (kVStep) dma16s(base + j0 * (NW * 1024), voff[0], vb + j * 1024);
-          else dma16s(base, voff[j0], vb + j * 1024);
-        }
-      }
-    } else {
-      issue_rows(vglob, koff, vb, kt);  // same geometry as K
-    }
-  };
+  auto issue_k = [&](unsigned char* kb, int kt) { issue_rows(kglob, koff, kb, kt, N, [](int row) { return KS::sw(row); }); };
+  // V: the same geometry.  Rows of v past the sequence's length may hold anything, and a zero probability does not
+  // silence a NaN in the product: the 16-bit tiles take the last valid row in their place (fp32 zeroes the operand).
+  auto issue_v = [&](unsigned char* vb, int kt) { issue_rows(vglob, voff, vb, kt, k16 ? L : N, vsw); };
 
   // Next tile index > cur allowed by `mask` (nullptr = every tile), or -1.  The mask word in use is kept in
   // a register, so LDS is read once per 32 tiles.
@@ -1225,8 +1242,8 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
         }
         need_v();
         if constexpr (k16) {
-          uint32_t va = (uint32_t)(uintptr_t)vt_lds + v_lane;
-          asm volatile("" : "+v"(va));
+          uint32_t va0 = (uint32_t)(uintptr_t)vt_lds + v_lane[0], va1 = (uint32_t)(uintptr_t)vt_lds + v_lane[1];
+          asm volatile("" : "+v"(va0), "+v"(va1));
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
             // a 16-key half in which no row of the wave has a non-zero probability adds nothing: with a
@@ -1235,8 +1252,10 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
 #pragma unroll
             for (int db = 0; db < G::kDB; ++db) {
               const int drow = db * 32 + lq;
-              u32x4 a = {0u, 0u, 0u, 0u};
-              if (D >= 32 || drow < D) a = lds_read16(va ^ ((kb * 4 + 2 * s) << 4), db * 32 * G::kVRow);
+              const u32x2_t a0 = lds_read8_tr(va0 ^ (db << 6), (kb * 32 + 16 * s) * G::kVRow);
+              const u32x2_t a1 = lds_read8_tr(va1 ^ (db << 6), (kb * 32 + 16 * s) * G::kVRow);
+              u32x4 a = {a0[0], a0[1], a1[0], a1[1]};
+              if (D < 32 && drow >= D) a = u32x4{0u, 0u, 0u, 0u};
               o[db] = mfma_16bit<T>(a, bp[s], o[db]);
             }
           }

@@ -80,11 +80,12 @@ int adsp_entmax_rows_bwd(const void* y, const void* dy, void* dx, int64_t rows, 
                          double alpha, void* stream);
 
 /*
- * Bytes of scratch the forward entry points need for these dimensions; 0 for fp32.  For the 16-bit types: a
- * key-major copy of V and, at head dims 64 and 128, the work counters, row-block flags and candidate streams of the
- * sparse-support kernel (up to 1024 slots of 51 KiB; sequences of up to 65536 keys) and a one-byte (fp8 e4m3) copy
- * of K.  The buffer must be 16-byte aligned device memory; its contents need not survive between calls, and two
- * calls that run at the same time need a buffer each.  For the block-mask variant pass Hq = Hkv = H.
+ * Bytes of scratch the forward entry points need for these dimensions; 0 for fp32 and for the head dims the
+ * sparse-support kernel does not serve (then `workspace` may be NULL).  For the 16-bit types at head dims 64 and 128:
+ * the work counters, row-block flags and candidate streams of the sparse-support kernel (up to 1024 slots of 51 KiB;
+ * sequences of up to 65536 keys) and a one-byte (fp8 e4m3) copy of K.  The buffer must be 16-byte aligned device
+ * memory; its contents need not survive between calls, and two calls that run at the same time need a buffer each.
+ * For the block-mask variant pass Hq = Hkv = H.
  */
 size_t adsp_attn_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
 
