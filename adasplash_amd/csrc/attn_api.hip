@@ -39,57 +39,6 @@ static const attn_fwd_fn kFwdTable[3][5][2] = {ADSP_FWD_TAG(f32), ADSP_FWD_TAG(b
 static const attn_bwd_fn kBwdTable[3][5] = {ADSP_BWD_TAG(f32), ADSP_BWD_TAG(bf16), ADSP_BWD_TAG(f16)};
 static int head_dim_slot(int D) { return D == 16 ? 0 : (D == 32 ? 1 : (D == 64 ? 2 : (D == 128 ? 3 : (D == 256 ? 4 : -1)))); }
 
-// Tile-wise key-major, MFMA-ordered copy of V for the 16-bit path.  Keys are cut in tiles of 64; a tile
-// is stored as one contiguous [D][64] block (so the kernel fetches it with contiguous kilobyte copies):
-//   vt[bh, kt, d, pos(n % 64)] = v[bh, n, d],  kt = n / 64,
-//   pos(16s + 8a + 4h + r) = 16s + 8h + 4a + r,  zero for n >= the sequence's valid length (so that
-//   whatever the caller left in the padding rows never meets an MFMA).
-// With this order a lane of the PV product reads its 8 keys {16s + 4h + r, 16s + 8 + 4h + r} of one
-// d row as one 16-byte LDS access.
-// A thread moves an 8-key x 8-d block: eight 16-byte loads (one key each), an 8 x 8 transpose of 16-bit values in
-// registers (32 byte permutes), eight 16-byte stores (one d row each).  A 64-key tile takes D threads.
-// `ctrl` (null, or the control words of the sparse-support forward, which ran before this kernel on the same stream):
-// the copy is only needed by the dense kernel, so it is skipped when that kernel has no row block to serve.
-__global__ __launch_bounds__(256) void vt_layout_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
-                                                        int N, int Npad, int D, const void* varlen, int varlen_bits,
-                                                        int heads, const uint32_t* ctrl) {
-  if (ctrl && ctrl[kCtrlFlagged] == 0u && ctrl[kCtrlAllDense] == 0u) return;
-  const int tiles_per_block = 256 / D;  // D <= 256
-  const int t = threadIdx.x % D;
-  const int kt = blockIdx.x * tiles_per_block + threadIdx.x / D;
-  if (kt >= Npad / 64) return;
-  const size_t bh = blockIdx.y;
-  int L = N;
-  if (varlen) {
-    const size_t b = bh / heads;
-    long long l = varlen_bits == 64 ? ((const long long*)varlen)[b] : (long long)((const int*)varlen)[b];
-    L = (int)(l < 0 ? 0 : (l > N ? N : l));
-  }
-  const int c = t & 7;    // output chunk: positions 8c .. 8c + 7 = keys 16s + 8a + 4h + r, s = c / 2, h = c % 2
-  const int dg = t >> 3;  // d values 8 dg .. 8 dg + 7
-  const uint16_t* vsrc = v + bh * (size_t)N * D + dg * 8;
-  const int key0 = kt * 64 + (c >> 1) * 16 + (c & 1) * 4;
-  u32x4 in[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int gk = key0 + (j >> 2) * 8 + (j & 3);
-    in[j] = u32x4{0u, 0u, 0u, 0u};
-    if (gk < L) in[j] = *reinterpret_cast<const u32x4*>(vsrc + (size_t)gk * D);
-  }
-  uint16_t* vdst = vt + bh * (size_t)D * Npad + (size_t)kt * 64 * D + (size_t)(dg * 8) * 64 + c * 8;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    u32x4 o;
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const uint32_t lo = in[2 * m][e >> 1], hi = in[2 * m + 1][e >> 1];
-      // (e even) low halves, (e odd) high halves of the two keys' dwords, packed key 2m low / key 2m + 1 high
-      o[m] = __builtin_amdgcn_perm(hi, lo, (e & 1) ? 0x07060302u : 0x05040100u);
-    }
-    *reinterpret_cast<u32x4*>(vdst + (size_t)e * 64) = o;
-  }
-}
-
 // e4m3 copy of K for the first walk of the sparse-support forward: [B * Hkv][Npad][D] bytes in the order of K, values
 // beyond the format's range saturated, rows from N on zero.  A thread converts 16 values.  Heads the probe has marked
 // as dense are skipped (`hints`: two words per head).
@@ -115,10 +64,6 @@ __global__ __launch_bounds__(256) void k8_layout_kernel(const uint16_t* __restri
   *reinterpret_cast<u32x4*>(k8 + (head * (size_t)Npad + row) * D + c * 16) = out;
 }
 
-static unsigned vt_layout_blocks(int Npad, int D) {  // 256 / D tiles of 64 keys per block
-  const int tiles = Npad / kBN, per_block = 256 / D;
-  return (unsigned)((tiles + per_block - 1) / per_block);
-}
 static int npad_of(int N) { return (N + kBN - 1) / kBN * kBN; }
 static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }
 static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
@@ -259,7 +204,6 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.q = q;
   p.k = k;
   p.v = v;
-  p.vt = nullptr;
   p.out = out;
   p.taus = taus;
   p.bmask = bmask;
@@ -401,9 +345,9 @@ extern "C" int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, voi
 }
 
 namespace adsp {
-// Workspace of the backward for the 16-bit types: the tile-wise transposed copies of k, q and dout, then -- for the
-// head dims the sparse-support dQ kernel serves -- its work counters, per-row-block flags and candidate streams (the
-// forward's layout without the copy of K).
+// Workspace of the backward for the 16-bit types, for the head dims the sparse-support kernels serve: their work
+// counters, per-row-block flags and candidate streams (the forward's layout without the copy of K).  (The dense
+// kernels need none: they read k, q and dout row-major and transpose in the LDS read.)
 struct BwdWorkspace {
   size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, part_off, part_bytes, total;
   int slots;  // 0: no sparse-support kernels for these dimensions
@@ -411,8 +355,8 @@ struct BwdWorkspace {
 static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
   BwdWorkspace w = {};
   if (dtype == ADSP_F32) return w;
-  w.copies_bytes = (size_t)B * (Hkv + 2 * (size_t)Hq) * D * npad_of(N) * 2;
-  w.total = w.copies_bytes;
+  w.copies_bytes = 0;
+  w.total = 0;
   if ((D == 64 || D == 128) && N <= 65536) {
     const long long items = (long long)B * Hq * mblocks_of(N);
     long long slots = (items + 7) / 8 * 8;
@@ -511,7 +455,6 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   p.k = k;
   p.v = v;
   p.dout = dout;
-  p.kt = p.qt = p.dot = nullptr;
   p.dq = dq;
   p.dk = dk;
   p.dv = dv;
@@ -549,13 +492,7 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   if (dtype != ADSP_F32) {
     w = bwd_workspace(B, Hq, Hkv, N, D, dtype);
     const size_t need = w.total;
-    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0) return ADSP_ERR_WORKSPACE;
-    uint16_t* kt = (uint16_t*)workspace;
-    uint16_t* qt = kt + (size_t)B * Hkv * D * p.Npad;
-    uint16_t* dot = qt + (size_t)B * Hq * D * p.Npad;
-    p.kt = kt;
-    p.qt = qt;
-    p.dot = dot;
+    if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0)) return ADSP_ERR_WORKSPACE;
     // Sparse-support dQ kernel first (alpha 1.5 / 2): it serves the row blocks whose supports are short and flags the
     // others for attn_bwd_dq_kernel below; the dK/dV kernel reads delta and 1 / sum p from whichever of the two wrote them.
     sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
@@ -588,17 +525,6 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
       }
       if (rc != 0) return ADSP_ERR_LAUNCH;
     }
-    // the transposed copies serve the dense kernels only: that of k the dQ kernel (skipped when the sparse-support
-    // kernel left it nothing), those of q and dout the dK/dV kernel (made further down when the sparse path is taken)
-    const unsigned gx = vt_layout_blocks(p.Npad, D);
-    hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hkv)), dim3(256), 0, s, (const uint16_t*)k, kt, N, p.Npad, D,
-                       varlen, varlen_bits, Hkv, (const uint32_t*)p.queue);
-    if (!sparse) {
-      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, qt, N, p.Npad, D,
-                         varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
-      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, dot, N, p.Npad,
-                         D, varlen, varlen_bits, Hq, (const uint32_t*)nullptr);
-    }
   }
   if (!sparse) {
     if (kBwdTable[dtype][head_dim_slot(D)](p, am, 3, s) != 0) return ADSP_ERR_LAUNCH;
@@ -628,13 +554,6 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     if (dtype == ADSP_BF16) rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, 1, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, 1, w.slots, s);
     else rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, 1, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, 1, w.slots, s);
     if (rc != 0) return ADSP_ERR_LAUNCH;
-    {
-      const unsigned gx = vt_layout_blocks(p.Npad, D);
-      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)q, (uint16_t*)const_cast<void*>(p.qt), N, p.Npad, D,
-                         varlen, varlen_bits, Hq, (const uint32_t*)p.queue2);
-      hipLaunchKernelGGL(vt_layout_kernel, dim3(gx, (unsigned)(B * Hq)), dim3(256), 0, s, (const uint16_t*)dout, (uint16_t*)const_cast<void*>(p.dot), N, p.Npad,
-                         D, varlen, varlen_bits, Hq, (const uint32_t*)p.queue2);
-    }
     if (kBwdTable[dtype][head_dim_slot(D)](p, am, 2, s) != 0) return ADSP_ERR_LAUNCH;
     if (w.part_bytes) {
       const long long threads = (long long)B * Hkv * N * (D / 8);

@@ -45,9 +45,15 @@ template <int AM> __device__ __forceinline__ void bwd_prob(float r, float c0, fl
 template <typename T, int D> struct BwdTiles {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
-  static constexpr int kTRow = G::k16 ? kBN * 2 : D * 4;  // 16-bit: a row of a transposed tile [D][64 keys]; fp32: of a [64][D] tile
-  using VS = Swz<kTRow>;
   static constexpr bool k16 = G::k16;
+  // Swizzle of a 16-bit tile that acc_block reads with the transposing LDS read (see attn_fwd_kernel's V tile): the four
+  // rows that the 16 lanes of a group address together fall into four different quarters of the banks.
+  static __device__ __forceinline__ int tsw(int row) {
+    constexpr int kC = KS::kC;
+    if constexpr (kC >= 8) return (2 * row) & ((kC >= 16 ? 16 : kC) - 1);
+    else if constexpr (kC == 4) return row & 2;
+    else return 0;
+  }
   static constexpr int kTile = G::kKTile;  // bytes of a [64][D] tile, in either orientation
   static constexpr int kNW = kBwdRows / 32;
   static constexpr int kSlots = k16 ? 3 : 2;  // tiles per pipeline stage
@@ -57,7 +63,10 @@ template <typename T, int D> struct BwdTiles {
   static constexpr int kMinWaves = G::kMinWaves < 2 ? G::kMinWaves : 2;
   static constexpr int kLoads = kTile / 1024;
 
-  // DMA of rows [row0, row0 + 64) of a row-major [N][D] tensor into a swizzled tile.
+  // DMA of rows [row0, row0 + 64) of a row-major [N][D] tensor into a swizzled tile; rows from `N` on (the tensor's end,
+  // or the sequence's for a tile that meets a product unmasked) are replaced by the last one before it.  kT: the tile
+  // is read by acc_block (transposing reads, their swizzle); else by dot_block.
+  template <bool kT = false>
   static __device__ __forceinline__ void issue_rows(const unsigned char* g, int row0, int N, unsigned char* lds, int wave,
                                                     int lane) {
     // the address is a wave-uniform base plus a 32-bit lane offset; for a whole tile the offset does not depend on the
@@ -69,7 +78,7 @@ template <typename T, int D> struct BwdTiles {
         const int j = j0 * kNW + wave;
         if (kLoads % kNW == 0 || j < kLoads) {
           const int P = j * 64 + lane;
-          const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
+          const int row = P / KS::kC, c = (P % KS::kC) ^ (kT ? tsw(row) : KS::sw(row));
           dma16s(base, (uint32_t)(row * G::kKRow + c * 16), lds + j * 1024);
         }
       }
@@ -80,24 +89,11 @@ template <typename T, int D> struct BwdTiles {
         const int j = j0 * kNW + wave;
         if (kLoads % kNW == 0 || j < kLoads) {
           const int P = j * 64 + lane;
-          const int row = P / KS::kC, c = (P % KS::kC) ^ KS::sw(row);
+          const int row = P / KS::kC, c = (P % KS::kC) ^ (kT ? tsw(row) : KS::sw(row));
           int gr = row0 + row;
           gr = gr < N ? gr : N - 1;  // rows past the end are masked by the caller
           dma16s(g, (uint32_t)gr * (uint32_t)G::kKRow + (uint32_t)(c * 16), lds + j * 1024);
         }
-      }
-    }
-  }
-  // DMA of one contiguous transposed tile ([D][64], as written by vt_layout_kernel) into a swizzled tile.
-  static __device__ __forceinline__ void issue_t(const unsigned char* gtile, unsigned char* lds, int wave, int lane) {
-    gtile = uniform_ptr(gtile);
-#pragma unroll
-    for (int j0 = 0; j0 < (kLoads + kNW - 1) / kNW; ++j0) {
-      const int j = j0 * kNW + wave;
-      if (kLoads % kNW == 0 || j < kLoads) {
-        const int P = j * 64 + lane;
-        const int row = P / VS::kC, c = (P % VS::kC) ^ VS::sw(row);
-        dma16s(gtile, (uint32_t)(row * kTRow + c * 16), lds + j * 1024);
       }
     }
   }
@@ -169,29 +165,27 @@ template <typename T, int D> struct BwdTiles {
     return acc;
   }
   // o^T[d][lane row] += sum over the 32 tile rows of block kb of  tile[row][d] * w[row][lane row], where
-  // w holds the lane's 16 values in the accumulator order of dot_block.  16-bit: `tile` is the transposed
-  // tile (its padding rows are zero); fp32: the row-major one, of which only the first `rows_valid` rows
-  // are used (padding rows of the caller's tensors may hold anything).
+  // w holds the lane's 16 values in the accumulator order of dot_block.  `tile` is row-major; only its first
+  // `rows_valid` rows count (padding rows of the caller's tensors may hold anything: fp32 zeroes the operand; the
+  // 16-bit tiles carry a valid row in their place, see issue_rows, and the callers select, not multiply, a zero weight
+  // for every pair outside the mask or the sequence, so such a row adds exactly nothing).  16-bit: the operand
+  // that runs along the tile's rows comes from two transposing reads per 16 rows -- in a group of 16 lanes, lane
+  // 4 r + c points at row (4 g + r [+ 8]) of the half block, g = lane / 32, and at columns 4 c .. 4 c + 3 of the group's
+  // 16 (groups 0 / 2: columns 0 .. 15 of a block of 32, groups 1 / 3: 16 .. 31), and receives column lane % 16 of four rows.
   template <bool kLean = false>
   static __device__ __forceinline__ void acc_block(f32x16 (&o)[G::kDB], const unsigned char* tile, int kb,
                                                    const float (&w)[16], int lq, int lh, int rows_valid) {
-    if constexpr (k16 && !kLean) {
+    if constexpr (k16) {
+      const int lane = lh * 32 + lq;
+      const int a4 = lane & 15, grp = lane >> 4, r = a4 >> 2, c = a4 & 3, dl = grp & 1;
+      uint32_t ta[2];
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        u32x4 b = {pack2<T>(w[8 * s], w[8 * s + 1]), pack2<T>(w[8 * s + 2], w[8 * s + 3]),
-                   pack2<T>(w[8 * s + 4], w[8 * s + 5]), pack2<T>(w[8 * s + 6], w[8 * s + 7])};
-#pragma unroll
-        for (int db = 0; db < G::kDB; ++db) {
-          const int drow = db * 32 + lq;
-          u32x4 a = {0u, 0u, 0u, 0u};
-          if (D >= 32 || drow < D) a = *reinterpret_cast<const u32x4*>(tile + VS::off(drow, kb * 4 + 2 * s + lh));
-          o[db] = mfma_16bit<T>(a, b, o[db]);
-        }
+      for (int h = 0; h < 2; ++h) {
+        const int x = 4 * lh + r + 8 * h;
+        ta[h] = (uint32_t)(uintptr_t)tile + (uint32_t)(x * G::kKRow + (((2 * dl + (c >> 1)) ^ tsw(x)) << 4) + (c & 1) * 8);
+        if (D < 32 && dl) ta[h] = (uint32_t)(uintptr_t)tile;  // (D = 16: these lanes' columns do not exist; their operand is zeroed)
       }
-    } else if constexpr (k16) {
-      // same addressing for the transposed tile: chunk 4 kb + 2 s + lh of row 32 db + lq
-      uint32_t ta = (uint32_t)(uintptr_t)tile + (uint32_t)(lq * kTRow + ((lh ^ VS::sw(lq)) << 4));
-      asm volatile("" : "+v"(ta));
+      asm volatile("" : "+v"(ta[0]), "+v"(ta[1]));
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         u32x4 b = {pack2<T>(w[8 * s], w[8 * s + 1]), pack2<T>(w[8 * s + 2], w[8 * s + 3]),
@@ -199,8 +193,10 @@ template <typename T, int D> struct BwdTiles {
 #pragma unroll
         for (int db = 0; db < G::kDB; ++db) {
           const int drow = db * 32 + lq;
-          u32x4 a = {0u, 0u, 0u, 0u};
-          if (D >= 32 || drow < D) a = lds_read16(ta ^ ((kb * 4 + 2 * s) << 4), db * 32 * kTRow);
+          const u32x2_t a0 = lds_read8_tr(ta[0] ^ (db << 6), (kb * 32 + 16 * s) * G::kKRow);
+          const u32x2_t a1 = lds_read8_tr(ta[1] ^ (db << 6), (kb * 32 + 16 * s) * G::kKRow);
+          u32x4 a = {a0[0], a0[1], a1[0], a1[1]};
+          if (D < 32 && drow >= D) a = u32x4{0u, 0u, 0u, 0u};
           o[db] = mfma_16bit<T>(a, b, o[db]);
         }
       }
@@ -332,8 +328,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T
 
   const unsigned char* kg = reinterpret_cast<const unsigned char*>(p.k) + kv_base * G::kKRow;
   const unsigned char* vg = reinterpret_cast<const unsigned char*>(p.v) + kv_base * G::kKRow;
-  const unsigned char* ktg =
-      k16 ? reinterpret_cast<const unsigned char*>(p.kt) + (size_t)(b * p.Hkv + kvh) * D * p.Npad * 2 : nullptr;
 
   auto next_tile = [&](int cur) -> int {
     int t = cur + 1;
@@ -352,7 +346,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T
     BT::issue_rows(kg, kt * kBN, N, a, wave, lane);
     BT::issue_rows(vg, kt * kBN, N, bb, wave, lane);
     if constexpr (k16) {
-      if (with_t) BT::issue_t(ktg + (size_t)kt * BT::kTile, c, wave, lane);
+      if (with_t) BT::template issue_rows<true>(kg, kt * kBN, L, c, wave, lane);  // K again, for the transposing reads of dQ
     }
   };
   auto tile_loop = [&](bool with_t, auto&& body) {
@@ -588,12 +582,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
       BT::issue_rows(qg, qt * kBN, N, a, wave, lane);
       if (pass >= 2 || !k16) BT::issue_rows(dog, qt * kBN, N, bb, wave, lane);
       if constexpr (k16) {
-        // transposed operand of the pass: dO^T for dV (pass 1 and the fused pass 3), Q^T for dK (pass 2;
-        // the fused pass takes it as a second transposed tile)
-        const size_t toff = bh * D * p.Npad * 2 + (size_t)qt * BT::kTile;
-        BT::issue_t(reinterpret_cast<const unsigned char*>(pass == 2 ? p.qt : p.dot) + toff, c, wave, lane);
+        // the operand of the pass that runs along the queries, in the format of the transposing reads: dO for dV
+        // (pass 1 and the fused pass 3), q for dK (pass 2; the fused pass takes it as a second such tile)
+        BT::template issue_rows<true>(pass == 2 ? qg : dog, qt * kBN, L, c, wave, lane);
         if constexpr (kFused) {
-          if (pass == 3) BT::issue_t(reinterpret_cast<const unsigned char*>(p.qt) + toff, d, wave, lane);
+          if (pass == 3) BT::template issue_rows<true>(qg, qt * kBN, L, d, wave, lane);
         }
       }
       // tau, 1 / sum p and delta of the tile's 64 queries: one 4-byte DMA per lane, an array per wave.

@@ -6,7 +6,6 @@ namespace adsp {
 
 struct AttnBwdParams {
   const void *q, *k, *v, *dout;
-  const void *kt, *qt, *dot;  // 16-bit path: tile-wise transposed copies of k, q, dout; unused for fp32
   void *dq, *dk, *dv;
   const float* taus;  // [B, Hq, N] thresholds of the forward, in z units
   float* delta;       // [B, Hq, N] written by the dQ kernel, read by the dK/dV kernel

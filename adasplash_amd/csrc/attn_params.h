@@ -18,7 +18,6 @@ struct AttnParams {
   const void* q;
   const void* k;
   const void* v;   // row-major V: the fp32 path walks it; every path gathers rows of it for the list-based output
-  const void* vt;  // 16-bit path: key-major permuted copy of V, [B*Hkv, D, Npad]
   void* out;
   float* taus;
   int32_t* bmask;
