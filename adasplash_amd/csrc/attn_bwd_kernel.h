@@ -14,8 +14,8 @@
 //                                                 pass 2 forms dX and dQ^T += K^T dX^T.
 //   dK/dV kernel, one workgroup per 128 keys, all query heads of the K/V head in turn:
 //                                                 pass 1 dV^T += dO^T P, pass 2 dK^T += Q^T dX.
-// The 16-bit path takes the transposed operands (K^T, dO^T, Q^T) from tile-wise transposed copies in the
-// layout of vt_layout_kernel, so that P / dX go from the accumulators straight into the next MFMA.
+// P / dX go from the accumulators straight into the next MFMA; the operands that run along the tile's rows (K^T, dO^T,
+// Q^T) come out of row-major tiles through the transposing LDS read (16-bit types, see acc_block).
 #pragma once
 #include <type_traits>
 #include "attn_kernel.h"

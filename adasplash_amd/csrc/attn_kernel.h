@@ -23,8 +23,9 @@
 //   D  p = [z - tau]_+^c0, out += P V over masked tiles, divided by sum p at the end.
 // In walks C and D the accumulator of the S^T MFMA is initialised with -tau, so z - tau costs no VALU op.
 //
-// The 16-bit path consumes V through a tile-wise key-major copy (vt_layout_kernel) so that the PV product
-// out^T = V^T P^T can take P^T straight from the S^T accumulators without an LDS round trip.
+// The PV product is taken as out^T = V^T P^T, so that P^T goes straight from the S^T accumulators into the next MFMA
+// without an LDS round trip; the 16-bit V tiles are row-major like K's and the operand V^T comes out of the
+// transposing LDS read (ds_read_b64_tr_b16).
 #pragma once
 #include <type_traits>
 #include "common.h"

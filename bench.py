@@ -40,13 +40,12 @@ MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.508e9, "c3": 0.4945e9, "c5": 0.621e9, "c2_
                               "c4_bwd": 24.9e9}  # c4_bwd: sparse dq kernel 2.41e9 + sparse dk/dv kernel 20.06e9 + reduction 2.42e9
 
 
-# The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is five launches: a
-# probe of the score distribution, the one-byte copy of K, the sparse-support kernel, the key-major copy of V and the
-# dense kernel, of which the last two return at once unless the sparse-support kernel left row blocks over (c3: the
-# probe marks every head dense, the copy of K and the sparse-support kernel step aside and the dense kernel does all
-# the work).
-FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + fp8 copy of K + this + V copy and attn_fwd_kernel on leftovers)",
-               "c3": "attn_fwd_kernel<bf16, 64, single step> (step = probe + sparse-support kernel stepping aside + V copy + this)",
+# The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
+# probe of the score distribution, the one-byte copy of K, the sparse-support kernel and the dense kernel, of which the
+# last returns at once unless the sparse-support kernel left row blocks over (c3: the probe marks every head dense, the
+# copy of K and the sparse-support kernel step aside and the dense kernel does all the work).
+FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + fp8 copy of K + this + attn_fwd_kernel on leftovers)",
+               "c3": "attn_fwd_kernel<bf16, 64, single step> (step = probe + sparse-support kernel stepping aside + this)",
                "c5": "attn_fwd_kernel<bf16, 64, generic alpha, candidate lists>"}
 
 

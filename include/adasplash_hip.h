@@ -112,7 +112,7 @@ int adsp_attn_v2_fwd(const void* q, const void* k, const void* v, void* out, flo
 /*
  * adsp_attn_v2_fwd without a workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
- * scratch memory (key-major copy of V, control words, flags, candidate streams and fp8 copy of K of the sparse-support kernel)
+ * scratch memory (control words, flags, candidate streams and fp8 copy of K of the sparse-support kernel)
  * lives in a device array inside the library, 64 MiB on every GPU the library runs on, held until the process ends;
  * problems whose adsp_attn_workspace_bytes() exceeds adsp_attn_v2_fwd_noalloc_max_bytes() are rejected with
  * ADSP_ERR_TOO_LARGE.  The call allocates and frees nothing and records no memset (the kernels clear what must start

@@ -51,7 +51,7 @@ def test_two_calls_in_a_row_match_the_entry_point_with_a_workspace(dtype, tol):
                                                              (1, 2, 2, 320, 64, [300], 10)]):
         q, k, v, varlen = _inputs(B, Hq, Hkv, N, D, dtype, seed=case)
         if case == 0:
-            q[1] *= 0.1  # a flat item: its heads go to the dense kernel, which reads the key-major copy of V
+            q[1] *= 0.1  # a flat item: its heads go to the dense kernel
         dev = [t.to(DEV) if t is not None else None for t in (q, k, v, varlen)]
         st_a, out_a, tau_a, bm_a = _call("noalloc", *dev, niter=niter)
         st_b, out_b, tau_b, bm_b = _call("workspace", *dev, niter=niter)
