@@ -213,16 +213,24 @@ def test_v_of_ones_returns_ones_and_linearity_in_v():
     assert (a + b - c).abs().max().item() < 1e-4
 
 
+@pytest.mark.parametrize("n", [32768, 16320, 16384, 8192])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_all_equal_scores_on_a_long_sequence_give_running_means(dtype):
+def test_all_equal_scores_on_a_long_sequence_give_running_means(dtype, n):
     """q = 0: every score of a row is equal, so every key lands in the top histogram bin and the row's
     probabilities are uniform; out_i is the mean of v_0..v_i.  With N = 32768 a lane counts 16384 entries in one
-    bin, which exercises the upper bit planes of the histogram counters (carries out of the per-tile adder tree)."""
+    bin, which exercises the upper bit planes of the histogram counters (carries out of the per-tile adder tree).
+    N = 16320 is the longest walk (255 tiles) that the short form of the counters (12 planes) serves, with 4080 entries
+    in one counter; N = 16384 is the first that takes the long form."""
     torch.manual_seed(0)
-    n = 32768
     q = torch.zeros(1, 1, n, 64).to(dtype)
     k = torch.randn(1, 1, n, 64).to(dtype)
     v = torch.randn(1, 1, n, 64).to(dtype)
-    out = run_v2(q, k, v, niter=1).double().cpu()
-    want = v.double().cumsum(2) / torch.arange(1, n + 1, dtype=torch.float64).view(1, 1, n, 1)
+    # (lengths that are no power of two go through varlen: the wrapper, like the reference, asks for a power of two)
+    N = 1 << (n - 1).bit_length()
+    if N != n:
+        pad = lambda t: torch.cat([t, torch.zeros(1, 1, N - n, 64, dtype=dtype)], dim=2)  # noqa: E731
+        q, k, v = pad(q), pad(k), pad(v)
+    varlen = torch.tensor([n], dtype=torch.int32) if N != n else None
+    out = run_v2(q, k, v, niter=1, varlen=varlen).double().cpu()[:, :, :n]
+    want = v[:, :, :n].double().cumsum(2) / torch.arange(1, n + 1, dtype=torch.float64).view(1, 1, n, 1)
     assert (out - want).abs().max().item() < (1e-4 if dtype == torch.float32 else 1e-2)
