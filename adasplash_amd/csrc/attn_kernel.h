@@ -999,12 +999,14 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
       tile_loop(mask_cur, false, [&](int kt, const unsigned char* kt_lds, const unsigned char*) {
         const uint32_t bits = block_bits(fine_cur, kt);
         float dmax0 = -INFINITY, dmax1 = -INFINITY;  // per 32-key block
-        if constexpr (k16 && AM != ATT_GEN) {
-          // 16-bit inputs: the sums run on pairs of scores rounded (towards zero) to f16 -- packed max, packed
-          // f16 sums over the tile (at most 16 terms of at most (sqrt(D) / (alpha - 1))^2 <= 1024 per half, added
+        if constexpr (k16 && AM == ATT_15) {
+          // 16-bit inputs, alpha = 1.5: the sums run on pairs of scores rounded (towards zero) to f16 -- packed max,
+          // packed f16 sums over the tile (at most 16 terms of at most (sqrt(D) / (alpha - 1))^2 <= 1024 per half, added
           // to the fp32 sums once per tile), and the sign bits for the support count: 3.5 VALU instructions per
           // score instead of 5.5.  The rounding moves f by a few 1e-4 relative, far inside the 16-bit output
-          // tolerance, and keeps {score > lower bound} a superset (negative values round up).  The sums use
+          // tolerance, and keeps {score > lower bound} a superset (negative values round up).  (alpha = 2 takes the
+          // fp32 sums below, which cost it no more: there a threshold that is 1e-4 off is harmless to the output but
+          // moves keys in and out of supports, and the backward weighs every member of a support alike.)  The sums use
           // v_pk_fma_f16 / v_pk_add_f16 and not the two-term dot product with fp32 accumulation: on this part a
           // wave's v_dot2 instructions and another wave's MFMAs exclude each other completely, while the other
           // vector instructions give up less than half of an MFMA's duration.
@@ -1067,7 +1069,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
           if (__builtin_amdgcn_ballot_w64(fmaxf(dmax0, dmax1) > dl) != 0ull && lane == 0) mark_tile(mask_new, kt);
         }
       });
-      if constexpr (k16 && AM != ATT_GEN) cnt_pos = n_seen - cnt_neg;
+      if constexpr (k16 && AM == ATT_15) cnt_pos = n_seen - cnt_neg;
       }
       if constexpr (AM == ATT_15) {
         a0 *= qs * qs;

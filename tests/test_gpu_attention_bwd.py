@@ -145,3 +145,37 @@ def test_backward_after_a_forward_on_candidate_lists(version, alpha, dtype, D):
     got, want = run_case(alpha, causal, 1, 2, 2, 1024, D, dtype, version=version, seed=3, scale=2.0)
     # dq and dk are linear in k and q, which are twice the size the 16-bit tolerance was set for
     check(got, want, dtype, tol_scale=1.0 if dtype == torch.float32 else 2.0)
+
+
+@pytest.mark.parametrize("sparse", ["1", "0"])
+@pytest.mark.parametrize("B,H,N,D,dtype,qscale,lens,causal,seed", [
+    (2, 2, 200, 64, torch.bfloat16, 0.3, [160, 185], False, 12),
+    (1, 2, 1024, 128, torch.float16, 1.0, None, False, 0),
+    (2, 2, 777, 64, torch.float16, 1.0, [640, 651], False, 33),
+])
+def test_sparsemax_gradients_on_flat_scores(sparse, B, H, N, D, dtype, qscale, lens, causal, seed):
+    """alpha = 2 weighs every member of a support alike in the backward (u = 1), so a threshold that is 1e-4 off --
+    harmless to the output -- moves a key in or out of a support and changes that row's gradient by O(1).  With flat
+    scores (small q) the supports are long and the dense kernels serve the rows (ADSP_SPARSE=0: all of them): their
+    solver walk keeps fp32 sums for alpha = 2 so that the threshold converges to the oracle's (it was 2e-4 off with the
+    packed f16 sums that alpha = 1.5 uses, and single rows of dq and dk were off by 1 to 5)."""
+    import os
+    old = os.environ.get("ADSP_SPARSE")
+    os.environ["ADSP_SPARSE"] = sparse
+    try:
+        g = torch.Generator().manual_seed(seed)
+        q = (qscale * torch.randn(B, H, N, D, generator=g)).to(dtype)
+        k = torch.randn(B, H, N, D, generator=g).to(dtype)
+        v = torch.randn(B, H, N, D, generator=g).to(dtype)
+        do = torch.randn(B, H, N, D, generator=g).to(dtype)
+        varlen = None if lens is None else torch.tensor(lens, dtype=torch.int32)
+        qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+        out = A.adasplash_v1(qg, kg, vg, alpha=2.0, is_causal=causal, varlen=None if varlen is None else varlen.to(DEV))
+        out.backward(do.to(DEV))
+        want = exact.dense_entmax_attention_grads(q, k, v, do, 2.0, causal, varlen)
+        check((qg.grad, kg.grad, vg.grad), want, dtype)
+    finally:
+        if old is None:
+            os.environ.pop("ADSP_SPARSE", None)
+        else:
+            os.environ["ADSP_SPARSE"] = old
