@@ -30,6 +30,24 @@ __device__ __forceinline__ void dma4s(const void* gbase, uint32_t off, void* lds
 }
 
 // sum over a group of LANES (8 or 16) adjacent lanes, left in every lane of the group
+// p[j] += a . b[j] over the eight 16-bit elements of a 16-byte chunk, j = 0 .. 3: sixteen two-term dot products with fp32
+// accumulation (the products of 16-bit values are exact in fp32, as with unpack + fma, at a quarter of the
+// instructions).  One block that ends in idle cycles: the instruction behind a v_dot2c must not overwrite one of its
+// sources (see dot2_chunk of the forward).
+template <typename T> __device__ __forceinline__ void dot8x4(float (&p)[4], u32x4 a, const u32x4 (&b)[4]);
+#define ADSP_DOT8X4(OP)                                                                                               \
+  asm volatile(OP " %0, %4, %8\n\t" OP " %1, %4, %12\n\t" OP " %2, %4, %16\n\t" OP " %3, %4, %20\n\t"                  \
+               OP " %0, %5, %9\n\t" OP " %1, %5, %13\n\t" OP " %2, %5, %17\n\t" OP " %3, %5, %21\n\t"                  \
+               OP " %0, %6, %10\n\t" OP " %1, %6, %14\n\t" OP " %2, %6, %18\n\t" OP " %3, %6, %22\n\t"                 \
+               OP " %0, %7, %11\n\t" OP " %1, %7, %15\n\t" OP " %2, %7, %19\n\t" OP " %3, %7, %23\n\ts_nop 3"           \
+               : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3])                                                        \
+               : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0][0]), "v"(b[0][1]), "v"(b[0][2]), "v"(b[0][3]),   \
+                 "v"(b[1][0]), "v"(b[1][1]), "v"(b[1][2]), "v"(b[1][3]), "v"(b[2][0]), "v"(b[2][1]), "v"(b[2][2]),     \
+                 "v"(b[2][3]), "v"(b[3][0]), "v"(b[3][1]), "v"(b[3][2]), "v"(b[3][3]))
+template <> __device__ __forceinline__ void dot8x4<bf16_t>(float (&p)[4], u32x4 a, const u32x4 (&b)[4]) { ADSP_DOT8X4("v_dot2c_f32_bf16"); }
+template <> __device__ __forceinline__ void dot8x4<f16_t>(float (&p)[4], u32x4 a, const u32x4 (&b)[4]) { ADSP_DOT8X4("v_dot2c_f32_f16"); }
+#undef ADSP_DOT8X4
+
 template <int LANES> __device__ __forceinline__ float group_sum(float x) {
   if constexpr (LANES == 16) {
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xf, 0xf, false));  // row_mirror
@@ -432,16 +450,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         const int r = r0 + grp;
         const bool row_live = wave_row0 + r < L;
         const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
-        float dov[8];  // the lane's eight columns of dO_i (rows past the valid length may hold anything: not read)
-        {
-          u32x4 raw = {0u, 0u, 0u, 0u};
-          if (row_live) raw = *reinterpret_cast<const u32x4*>(dorows + (size_t)r * (D * 2));
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            dov[2 * i] = unpack_lo<T>(raw[i]);
-            dov[2 * i + 1] = unpack_hi<T>(raw[i]);
-          }
-        }
+        u32x4 dov = {0u, 0u, 0u, 0u};  // the lane's eight columns of dO_i (rows past the valid length may hold anything: not read)
+        if (row_live) dov = *reinterpret_cast<const u32x4*>(dorows + (size_t)r * (D * 2));
         float acc_a[8], acc_b[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -464,12 +474,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
               kk[j] = *reinterpret_cast<const u32x4*>(krows + (size_t)key * (D * 2));
             }
           }
+          static_assert(kDepth == 4, "dot8x4 takes four members");
+          float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
+          dot8x4<T>(part, dov, vv);
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
-            float part = 0.f;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) part = fmaf(dov[2 * i], unpack_lo<T>(vv[j][i]), fmaf(dov[2 * i + 1], unpack_hi<T>(vv[j][i]), part));
-            const float dp = group_sum<kLPR>(part);  // dO_i . v_j, in every lane of the group
+            const float dp = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
             float pr, u;
             bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
             zsum += pr;
@@ -955,16 +965,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         const int r = r0 + grp;
         const int key = wave_row0 + r;
         const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
-        float vj[8];
-        {
-          u32x4 raw = {0u, 0u, 0u, 0u};
-          if (key < L) raw = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            vj[2 * i] = unpack_lo<T>(raw[i]);
-            vj[2 * i + 1] = unpack_hi<T>(raw[i]);
-          }
-        }
+        u32x4 vj = {0u, 0u, 0u, 0u};  // the lane's eight columns of v_j
+        if (key < L) vj = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
         float acc_v[8], acc_k[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -990,6 +992,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
               zi[j] = zinv_rows[qidx];
             }
           }
+          static_assert(kDepth == 4, "dot8x4 takes four members");
+          float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
+          dot8x4<T>(part, vj, dd);
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
             float dof[8];
@@ -998,10 +1003,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
               dof[2 * i] = unpack_lo<T>(dd[j][i]);
               dof[2 * i + 1] = unpack_hi<T>(dd[j][i]);
             }
-            float part = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) part = fmaf(dof[i], vj[i], part);
-            const float dp = group_sum<kLPR>(part);  // dO_i . v_j, in every lane of the group
+            const float dp = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
             float pr, u;
             bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
             const float ph = pr * zi[j], dx = u * (dp - dl[j]);
