@@ -46,11 +46,13 @@ template <typename T, int D> struct BwdTiles {
   using G = TileGeo<T, D>;
   using KS = Swz<G::kKRow>;
   static constexpr bool k16 = G::k16;
-  // Swizzle of a 16-bit tile that acc_block reads with the transposing LDS read (see attn_fwd_kernel's V tile): the four
-  // rows that the 16 lanes of a group address together fall into four different quarters of the banks.
+  // Swizzle of a 16-bit tile that acc_block reads with the transposing LDS read (see attn_fwd_kernel's V tile): the
+  // four rows times two column blocks that two groups of 16 lanes address together fall into eight different eighths
+  // of the banks.
   static __device__ __forceinline__ int tsw(int row) {
     constexpr int kC = KS::kC;
-    if constexpr (kC >= 8) return (2 * row) & ((kC >= 16 ? 16 : kC) - 1);
+    if constexpr (kC >= 16) return (4 * row) & 15;
+    else if constexpr (kC == 8) return (2 * row) & 7;
     else if constexpr (kC == 4) return row & 2;
     else return 0;
   }
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((dq_waves<T
   const int n_blk = (N + kBwdRows - 1) / kBwdRows;
   const int group = p.Hq / p.Hkv;
   int bkv, mi, hg;
-  if (!xcd_block_map(p.B * p.Hkv, n_blk, group, p.causal != 0, bkv, mi, hg)) return;
+  if (!xcd_block_map(p.B * p.Hkv, n_blk, group, p.causal != 0, 2ll * N * D * G::kEB, bkv, mi, hg)) return;  // (K and V of a head)
   const int mblk = n_blk - 1 - mi;  // the longest causal rows first; a group's heads side by side
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int h = kvh * group + hg;
@@ -514,7 +516,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((BwdTiles<T
   const int N = p.N;
   int bkv, nblk;  // early key blocks have the most causal work and come first
   int member_unused;
-  if (!xcd_block_map(p.B * p.Hkv, (N + kBwdRows - 1) / kBwdRows, 1, p.causal != 0, bkv, nblk, member_unused)) return;
+  // (the key blocks of a K/V head stream q and dout of all its query heads)
+  if (!xcd_block_map(p.B * p.Hkv, (N + kBwdRows - 1) / kBwdRows, 1, p.causal != 0, 2ll * (p.Hq / p.Hkv) * N * D * G::kEB, bkv, nblk, member_unused)) return;
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int group = p.Hq / p.Hkv;
   // behind the sparse-support dK/dV kernel: only the key blocks it flagged (all of them when it stepped aside)

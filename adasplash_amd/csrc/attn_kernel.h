@@ -238,7 +238,7 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   const int n_mblk = (p.N + BM - 1) / BM;
   const int group = p.Hq / p.Hkv;
   int bkv, mi, hg;
-  if (!xcd_block_map(p.B * p.Hkv, n_mblk, group, p.causal != 0, bkv, mi, hg)) return;
+  if (!xcd_block_map(p.B * p.Hkv, n_mblk, group, p.causal != 0, 2ll * p.N * D * G::kEB, bkv, mi, hg)) return;  // (K and V of a head)
   const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
   const int h = kvh * group + hg;
   const int mblk = n_mblk - 1 - mi;
@@ -321,14 +321,18 @@ __attribute__((amdgpu_waves_per_eu(fwd_min_waves<T, D, kMulti>(), (fwd_min_waves
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
   constexpr int kKOffs = kKStep ? 1 : kKPer;
   uint32_t koff[kKOffs], voff[kKOffs];
-  // The 16-bit V tile has a swizzle of its own, made for the transposing reads of the output product: the four rows
-  // that the 16 lanes of a group address together (keys x .. x + 3, 32 bytes of each) must fall into four different
-  // quarters of the 128 bytes that the banks serve per cycle, i.e. differ in bits 1 and 2 of their chunk position.
-  // Its period (4 rows) divides that of the K tile's, so the scalar-base stepping of the loads holds for both.
+  // The 16-bit V tile has a swizzle of its own, made for the transposing reads of the output product.  Two groups of 16
+  // lanes are served together: four rows (keys x .. x + 3) times two 32-byte column blocks, which must fall into
+  // eight different 32-byte eighths of the 256 bytes that the 64 banks serve per cycle.  Rows 256 bytes or more apart
+  // start in the same bank, so there the swizzle moves row r by 4 r chunks; rows of 128 bytes alternate between the
+  // halves of the banks by themselves and are moved by 2 r (measured: no conflict cycles either way, against a
+  // fifth of the LDS cycles with 2 r at 256 bytes).  Its period (4 rows) divides that of the K tile's, so the
+  // scalar-base stepping of the loads holds for both.
   auto vsw = [](int row) -> int {
     if constexpr (k16) {
       constexpr int kC = KS::kC;
-      if constexpr (kC >= 8) return (2 * row) & ((kC >= 16 ? 16 : kC) - 1);
+      if constexpr (kC >= 16) return (4 * row) & 15;
+      else if constexpr (kC == 8) return (2 * row) & 7;
       else if constexpr (kC == 4) return row & 2;
       else return 0;
     } else {

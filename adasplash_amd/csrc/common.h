@@ -113,9 +113,14 @@ __device__ __forceinline__ int wave_sum_i(int v) {
 // few of them, a set takes as many heads as give about two blocks per slot and runs them longest block first
 // over all its heads: started in that order, the short blocks fill the slots the long ones leave, where head
 // after head the last head's longest block would start when the others are almost through.
-// `blocks` = blocks per (head, member of its group), `group` = query heads per K/V head; returns false for the
-// padding blocks of the grid, else the K/V head, the block index and the member.
-__device__ __forceinline__ bool xcd_block_map(int units, int blocks, int group, bool balance, int& unit, int& blk, int& member) {
+// `blocks` = blocks per (head, member of its group), `group` = query heads per K/V head, `unit_bytes` = what the
+// blocks of one K/V head stream through L2 (they share it while they run side by side): a set never takes more heads
+// than bring 8 MB of that, twice an XCD's L2 -- with more, the blocks of a head that are in flight together become
+// too few to share their tiles, and on long sequences that costs more than the balance gains (dK/dV kernel on
+// B=8, Hkv=8, group 4, N=8192, D=128: 10.1 ms with sets of four heads, 7.5 ms head after head).  Returns false for
+// the padding blocks of the grid, else the K/V head, the block index and the member.
+__device__ __forceinline__ bool xcd_block_map(int units, int blocks, int group, bool balance, long long unit_bytes, int& unit, int& blk,
+                                              int& member) {
   const int inner = blocks * group;
   const int x = (int)(blockIdx.x & 7);
   const long long seq = (long long)(blockIdx.x >> 3);
@@ -132,7 +137,11 @@ __device__ __forceinline__ bool xcd_block_map(int units, int blocks, int group, 
   const int upx = units / 8;  // heads of this XCD
   if (seq >= (long long)upx * inner) return false;
   constexpr int kSetBlocks = 256;  // two blocks for each of 32 CUs x 4 resident blocks
+  constexpr long long kSetBytes = 8ll << 20;
   int g = balance ? (kSetBlocks + inner - 1) / inner : 1;
+  const long long by_bytes = unit_bytes > 0 ? kSetBytes / unit_bytes : (long long)upx;
+  g = g < by_bytes ? g : (int)by_bytes;
+  g = g < 1 ? 1 : g;
   g = g < upx ? g : upx;
   const int set = (int)(seq / ((long long)g * inner));
   const int s = (int)(seq - (long long)set * g * inner);
