@@ -391,12 +391,14 @@ __global__ __launch_bounds__(256) void bwd_ctrl_clear_kernel(uint32_t* ctrl2, co
 }
 
 // dK, dV = sum over the query heads of a K/V head of the sparse-support kernel's fp32 partial rows; key blocks left to
-// attn_bwd_dkdv_kernel are skipped (that kernel writes them).  A thread adds up 8 columns of one key row.
+// attn_bwd_dkdv_kernel are skipped (that kernel writes them).  A thread adds up 8 columns of one key row.  Rows past
+// the valid length are zeros and their partial rows are not read (the key blocks that lie wholly in the padding have
+// none).
 typedef float reduce_f32x4 __attribute__((ext_vector_type(4)));
 template <typename T>
 __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restrict__ dk_part, const float* __restrict__ dv_part,
                                                          void* dk, void* dv, const int32_t* kv_flags, const uint32_t* ctrl2,
-                                                         int B, int Hq, int Hkv, int N, int D) {
+                                                         const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D) {
   if (ctrl2[kCtrlAllDense] != 0u) return;
   const int per_row = D / 8;
   const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -406,10 +408,15 @@ __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restric
   const int row = (int)(rg % N), bkv = (int)(rg / N);
   if (kv_flags[(size_t)bkv * ((N + kMaskRows - 1) / kMaskRows) + row / kMaskRows] != 0) return;
   const int group = Hq / Hkv, b = bkv / Hkv, kvh = bkv % Hkv;
+  long long L = N;
+  if (varlen) {
+    L = varlen_bits == 64 ? ((const long long*)varlen)[b] : (long long)((const int*)varlen)[b];
+    L = L < 0 ? 0 : (L > N ? N : L);
+  }
   float sk[8], sv[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) sk[i] = sv[i] = 0.f;
-  for (int g = 0; g < group; ++g) {
+  for (int g = 0; g < (row < L ? group : 0); ++g) {
     const size_t at = (((size_t)(b * Hq + kvh * group + g) * N) + row) * D + c * 8;
     const reduce_f32x4 k0 = *reinterpret_cast<const reduce_f32x4*>(dk_part + at), k1 = *reinterpret_cast<const reduce_f32x4*>(dk_part + at + 4);
     const reduce_f32x4 v0 = *reinterpret_cast<const reduce_f32x4*>(dv_part + at), v1 = *reinterpret_cast<const reduce_f32x4*>(dv_part + at + 4);
@@ -560,10 +567,10 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
       const dim3 grid((unsigned)((threads + 255) / 256));
       if (dtype == ADSP_BF16)
         hipLaunchKernelGGL(dkdv_reduce_kernel<bf16_t>, grid, dim3(256), 0, s, (const float*)p.dk_part, (const float*)p.dv_part, dk, dv,
-                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, B, Hq, Hkv, N, D);
+                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, varlen, varlen_bits, B, Hq, Hkv, N, D);
       else
         hipLaunchKernelGGL(dkdv_reduce_kernel<f16_t>, grid, dim3(256), 0, s, (const float*)p.dk_part, (const float*)p.dv_part, dk, dv,
-                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, B, Hq, Hkv, N, D);
+                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, varlen, varlen_bits, B, Hq, Hkv, N, D);
     }
   }
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;

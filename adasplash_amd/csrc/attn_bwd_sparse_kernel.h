@@ -644,16 +644,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
     const int qi = m0 + wave * 32 + lq;
 
-    if (m0 >= L) {  // key block entirely inside the padding: zero gradient (nothing else writes these rows)
-      const int rows = (N - m0) < BM ? (N - m0) : BM;
-      float* o0 = p.dk_part + qo_base + (size_t)m0 * D;
-      float* o1 = p.dv_part + qo_base + (size_t)m0 * D;
-      for (int i = tid; i < rows * D; i += SG::kThreads) {
-        o0[i] = 0.f;
-        o1[i] = 0.f;
-      }
-      continue;
-    }
+    if (m0 >= L) continue;  // key block entirely inside the padding: dkdv_reduce_kernel writes its zeros without reading partial rows
 
     if (s_skip) {
       if (tid == 0) {
