@@ -187,6 +187,13 @@ static bool sparse_enabled() {
   return !(e && strcmp(e, "0") == 0);
 }
 
+// ADSP_BWD_STREAMS=0 in the environment makes the sparse-support dK/dV kernel walk for itself instead of taking the
+// dQ kernel's streams (for comparisons and tests).
+static bool bwd_streams_enabled() {
+  const char* e = getenv("ADSP_BWD_STREAMS");
+  return !(e && strcmp(e, "0") == 0);
+}
+
 static int attn_common(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
                        const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
                        double alpha, int is_causal, int niter, int use_hist, void* workspace, size_t workspace_bytes,
@@ -349,8 +356,9 @@ namespace adsp {
 // counters, per-row-block flags and candidate streams (the forward's layout without the copy of K).  (The dense
 // kernels need none: they read k, q and dout row-major and transpose in the LDS read.)
 struct BwdWorkspace {
-  size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, part_off, part_bytes, total;
-  int slots;  // 0: no sparse-support kernels for these dimensions
+  size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, part_off, part_bytes, streams_off, dir_off, total;
+  int slots;       // 0: no sparse-support kernels for these dimensions
+  int dir_stride;  // offsets per stream of the hand-over table
 };
 static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
   BwdWorkspace w = {};
@@ -371,7 +379,11 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     w.kvflags_off = align256(w.queue2_off + 256 + ((size_t)B * Hkv + 1) * 8);
     w.part_off = align256(w.kvflags_off + (size_t)B * Hkv * mblocks_of(N) * 4);
     w.part_bytes = (size_t)B * Hq * N * D * 4;
-    w.total = w.part_off + 2 * w.part_bytes;
+    // the dQ kernel's streams, kept per (row block, wave) for the dK/dV kernel, and where their 32-key blocks start
+    w.streams_off = align256(w.part_off + 2 * w.part_bytes);
+    w.dir_stride = (mblocks_of(N) * 4 + 2) / 2 * 2;
+    w.dir_off = align256(w.streams_off + (size_t)items * kSparseSlotBytes);  // (a slot = the streams of four waves)
+    w.total = w.dir_off + align256((size_t)items * 4 * w.dir_stride * 2);
   }
   return w;
 }
@@ -491,6 +503,9 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   p.kv_flags = nullptr;
   p.dk_part = nullptr;
   p.dv_part = nullptr;
+  p.streams = nullptr;
+  p.stream_dir = nullptr;
+  p.dir_stride = 0;
   const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
   bool sparse = false;
   BwdWorkspace w = {};
@@ -509,6 +524,11 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
       p.hints = p.queue + 64;
       p.block_flags = (int32_t*)(ws + w.flags_off);
       p.events = ws + w.events_off;
+      if (bwd_streams_enabled()) {
+        p.streams = ws + w.streams_off;
+        p.stream_dir = (uint16_t*)(ws + w.dir_off);
+        p.dir_stride = w.dir_stride;
+      }
       AttnParams pp = {};  // what the probe reads: q, k, lengths, dimensions, scale and the control words it clears
       pp.q = q;
       pp.k = k;
@@ -558,8 +578,9 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
     hipLaunchKernelGGL(bwd_ctrl_clear_kernel, dim3((unsigned)clear_blocks), dim3(256), 0, s, p.queue2, (const uint32_t*)p.hints, B * Hkv,
                        p.kv_flags, n_flags);
     int rc;
-    if (dtype == ADSP_BF16) rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, 1, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, 1, w.slots, s);
-    else rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, 1, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, 1, w.slots, s);
+    const int kind = p.streams ? 2 : 1;  // from the dQ kernel's streams, or with a walk of its own
+    if (dtype == ADSP_BF16) rc = D == 64 ? launch_attn_bwd_sparse_bf16_d64(p, am, kind, w.slots, s) : launch_attn_bwd_sparse_bf16_d128(p, am, kind, w.slots, s);
+    else rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, kind, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, kind, w.slots, s);
     if (rc != 0) return ADSP_ERR_LAUNCH;
     if (kBwdTable[dtype][head_dim_slot(D)](p, am, 2, s) != 0) return ADSP_ERR_LAUNCH;
     if (w.part_bytes) {

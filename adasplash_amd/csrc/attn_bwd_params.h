@@ -31,6 +31,11 @@ struct AttnBwdParams {
   int32_t* kv_flags;  // [B, Hkv, n_mblk] 1 = key block left to attn_bwd_dkdv_kernel
   float* dk_part;
   float* dv_part;
+  // hand-over of the supports from the dQ kernel to the dK/dV kernel (null: the dK/dV kernel walks for itself): the dQ
+  // kernel's streams kept per (row block, wave) instead of per workgroup, and per stream the offsets of the 32-key blocks
+  unsigned char* streams;  // [B, Hq, n_mblk, waves, stream capacity] (score - threshold, key | row << 20) pairs
+  uint16_t* stream_dir;    // [B, Hq, n_mblk, waves, dir_stride]: entry k = first stream entry with key >= 32 k
+  int dir_stride;          // 4 n_mblk + 1 offsets, rounded up to an even count
 };
 
 }  // namespace adsp

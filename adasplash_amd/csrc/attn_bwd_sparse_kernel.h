@@ -301,7 +301,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // and row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
     float* const ring = reinterpret_cast<float*>(lds_all + SG::kStages * G::kKTile + wave * SG::kRingBytes);
     uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
-    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
+    // (with the hand-over to the dK/dV kernel the stream has a place of its own per row block and wave, and stays)
+    const size_t stream_id = ((size_t)(b * p.Hq + h) * n_mblk + mblk) * NW + wave;
+    uint2* const stream = p.streams ? reinterpret_cast<uint2*>(p.streams) + stream_id * (size_t)kSparseStreamCap
+                                    : reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
     int ring_n = 0, stream_n = 0;  // wave-uniform
     // (kt: the tile being worked on; a stream that fills faster than the tiles go by will not last: give up early)
     auto flush = [&](int parity, int kt) {
@@ -410,6 +413,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         const int e = j * 64 + lane;
         ent[j] = uint2{0u, 0u};
         if (e < stream_n) ent[j] = stream[e];
+      }
+      if (p.stream_dir) {
+        // The walk went through the key tiles in order and the ring keeps the order of its events, so the stream is
+        // sorted by 16-key half block.  dir[k] = index of the first entry whose key is >= 32 k (k = 0 .. 4 n_mblk; the last
+        // one is the stream's length): the entry that opens a new 32-key block writes the offsets of the blocks it
+        // skipped and its own, and the position behind the last entry closes the table.
+        static_assert(kPer * 64 > SG::kListCap, "the position behind the last entry belongs to one of the groups");
+        uint16_t* const dir = p.stream_dir + stream_id * (size_t)p.dir_stride;
+        const int n32 = n_mblk * (BM / 32);
+        int carry = -1;  // 32-key block of the entry before this group of 64
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          if (j * 64 <= stream_n) {
+            const int e = j * 64 + lane;
+            const int kb = e < stream_n ? (int)((ent[j].y & 0xffffu) >> 5) : n32;
+            int prev = __shfl_up(kb, 1, 64);
+            prev = lane == 0 ? carry : prev;
+            if (e <= stream_n)
+              for (int k = prev + 1; k <= kb; ++k) dir[k] = (uint16_t)e;
+            carry = __builtin_amdgcn_readlane(kb, 63);
+          }
+        }
       }
 #pragma unroll
       for (int j = 0; j < kPer; ++j) {
@@ -1060,10 +1085,323 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 
 
 
-// Workgroups to launch: as many as fit the device at once (each owns one stream slot), at most `max_slots`.
-template <typename T, int D, int AM, bool kKeys> static int launch_attn_bwd_sparse_one(const AttnBwdParams& p, int max_slots, hipStream_t s) {
+// dK and dV from the supports the dQ kernel found (16-bit inputs, alpha = 1.5 / 2, head dims 64 / 128): the same work as
+// attn_bwd_dkdv_sparse_kernel without its score walk.  The dQ kernel leaves the stream of every (row block, wave) in
+// place -- (score - threshold, key | row) pairs sorted by 16-key half block -- with a table of where each 32-key block
+// starts.  A workgroup serves one (key block, query head); each of its waves owns 32 keys, copies the pieces of all
+// streams of the head that hold its keys (row blocks from its own on with a causal mask) into a stream of its own, as
+// (score - threshold, query | key << 20) pairs, and from there on does what the walking kernel does: a counting sort by
+// key into lists in LDS, and per key the sums over its queries.  A wave that has more members than its lists hold works
+// them off in parts; the waves of a workgroup share nothing and do not wait for each other.  A key block one of whose
+// row blocks the dQ kernel gave up (no stream) is flagged for attn_bwd_dkdv_kernel with all its heads.
+template <typename T, int D, int AM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE_WAVES, ADSP_SPARSE_WAVES))) void attn_bwd_dkdv_stream_kernel(AttnBwdParams p) {
+  using G = TileGeo<T, D>;
   using SG = SparseGeo<T, D>;
-  auto kern = kKeys ? attn_bwd_dkdv_sparse_kernel<T, D, AM> : attn_bwd_dq_sparse_kernel<T, D, AM>;
+  static_assert(G::k16, "16-bit element types only");
+  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  constexpr int NW = SG::kNW, BM = SG::kBM;
+  __shared__ __align__(16) unsigned char lds_all[NW * SG::kWaveLds];
+  __shared__ int s_item, s_skip;
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int N = p.N;
+  const int n_mblk = (N + BM - 1) / BM;
+  const int group = p.Hq / p.Hkv;
+  const long long total = (long long)p.B * p.Hkv * n_mblk * group;
+  const long long per_xcd = (total + 7) / 8;
+  const float qs = p.qscale;
+
+  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all key blocks
+    const int units = p.B * p.Hkv;
+    int unmarked = 0;
+    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints2[2 * u] < (1u << 20) ? 1 : 0;
+    if (__syncthreads_count(unmarked) == 0) {
+      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue2[kCtrlAllDense] = 1u;
+      return;
+    }
+  }
+  int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
+  for (;;) {
+    __syncthreads();  // the previous item is done with s_item
+    if (tid == 0) {
+      int got = -1;
+      while (queues_tried < 8) {
+        const int x = ((int)(blockIdx.x & 7) + queues_tried) & 7;
+        const long long i = (long long)atomicAdd(&p.queue2[x], 1u);
+        const long long logical = (long long)x * per_xcd + i;
+        if (i < per_xcd && logical < total) {
+          got = (int)logical;
+          break;
+        }
+        ++queues_tried;
+      }
+      s_item = got;
+      s_skip = 0;
+      if (got >= 0) {  // the K/V head of the key block, as decoded below: marked dense by the probe?
+        int unit = got / (group * n_mblk);
+        const int units = p.B * p.Hkv;
+        if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
+        s_skip = __hip_atomic_load(p.hints2 + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (1u << 20) ? 1 : 0;
+      }
+    }
+    __syncthreads();
+    const int logical = s_item;
+    if (logical < 0) break;
+
+    // ---- item -> (batch, kv head, key block, head in group), in the order of the dQ kernel's row blocks ---------
+    const int hg = logical % group;
+    const int mblk = (logical / group) % n_mblk;  // key block: with a causal mask the first ones see the most queries
+    int bkv = logical / (group * n_mblk);
+    {
+      const int units = p.B * p.Hkv;
+      if (units % 8 == 0) bkv = (bkv % (units / 8)) * 8 + bkv / (units / 8);
+    }
+    const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
+    const int h = kvh * group + hg;
+    const int m0 = mblk * BM;
+    int L = N;
+    if (p.varlen) {
+      long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
+      L = (int)(l < 0 ? 0 : (l > N ? N : l));
+    }
+    if (m0 >= L) continue;  // key block entirely inside the padding: dkdv_reduce_kernel writes its zeros
+    // a key block that any query head gives up goes to attn_bwd_dkdv_kernel with all its heads
+    int32_t* const flag = p.kv_flags + ((size_t)(b * p.Hkv + kvh) * n_mblk + mblk);
+    const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
+    const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
+    // the row blocks whose queries can hold the block's keys in their supports
+    const int rb_lo = p.causal ? mblk : 0, rb_hi = (L - 1) / BM;
+    {  // no stream where the dQ kernel gave a row block up
+      const int32_t* const dq_flags = p.block_flags + (size_t)(b * p.Hq + h) * n_mblk;
+      int any = s_skip;
+      for (int rb = rb_lo + tid; rb <= rb_hi; rb += SG::kThreads) any |= dq_flags[rb] != 0 ? 1 : 0;
+      if (__syncthreads_or(any)) {
+        if (tid == 0) {
+          *flag = 1;
+          atomicAdd(&p.queue2[kCtrlFlagged], 1u);
+        }
+        continue;
+      }
+    }
+    const int wave_row0 = m0 + wave * 32;
+    const int k32 = wave_row0 / 32;
+    const int n_pairs = (rb_hi - rb_lo + 1) * NW;  // (row block, wave of the dQ kernel) in order
+    const size_t head_stream0 = (size_t)(b * p.Hq + h) * n_mblk * NW;  // first stream of the head
+    const uint2* const src_streams = reinterpret_cast<const uint2*>(p.streams) + head_stream0 * (size_t)kSparseStreamCap;
+    const uint16_t* const src_dir = p.stream_dir + head_stream0 * (size_t)p.dir_stride + k32;
+    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
+
+    unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
+    float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap scores minus the threshold
+    uint16_t* const lkey = reinterpret_cast<uint16_t*>(wave_lds + SG::kListCap * 4);         // their queries
+    uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 6);     // 32 counters
+    uint32_t* const row_start = row_cnt + 32;                                                // 33 offsets
+    // while the pieces are copied the lists' room holds, per piece of the batch: entries up to and including it, where
+    // it starts among the head's streams, and the first query row of its stream
+    uint32_t* const pc_incl = reinterpret_cast<uint32_t*>(wave_lds);
+    uint32_t* const pc_src = pc_incl + 64;
+    uint32_t* const pc_row = pc_src + 64;
+    static_assert(SG::kListCap * 4 >= 3 * 64 * 4, "room for the batch table");
+
+    int cursor = 0;  // next piece (wave-uniform)
+    for (int seg = 0;; ++seg) {
+      int stream_n = 0;  // wave-uniform
+      while (cursor < n_pairs) {
+        const int pi = cursor + lane;
+        uint32_t len = 0u, src = 0u, row0 = 0u;
+        if (pi < n_pairs) {
+          const int rb = rb_lo + pi / NW, w = pi % NW;
+          const size_t sid = (size_t)rb * NW + w;
+          uint32_t lo = src_dir[sid * (size_t)p.dir_stride], hi = src_dir[sid * (size_t)p.dir_stride + 1];
+          hi = hi < (uint32_t)SG::kListCap ? hi : (uint32_t)SG::kListCap;  // (what the dQ kernel wrote lies within these bounds)
+          lo = lo < hi ? lo : hi;
+          len = hi - lo;
+          src = (uint32_t)(sid * (size_t)kSparseStreamCap) + lo;
+          row0 = (uint32_t)(rb * BM + w * 32);
+        }
+        const int incl = wave_scan_i((int)len);
+        // the pieces of this batch that still fit (the sums grow with the lane: a run of lanes from 0 on)
+        const unsigned long long fm = __builtin_amdgcn_ballot_w64(pi < n_pairs && stream_n + incl <= SG::kListCap);
+        const int m = __builtin_popcountll(fm);
+        if (m == 0) break;  // (the stream is not empty then: a single piece is no longer than a list)
+        const int batch = __builtin_amdgcn_readlane(incl, m - 1);
+        __builtin_amdgcn_wave_barrier();
+        if (lane < m) {
+          pc_incl[lane] = (uint32_t)incl;
+          pc_src[lane] = src;
+          pc_row[lane] = row0;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int e0 = 0; e0 < batch; e0 += 64) {
+          const int e = e0 + lane;
+          if (e < batch) {
+            int a = 0, z = m - 1;  // the piece that holds entry e: the first one whose running sum exceeds e
+            while (a < z) {
+              const int mid = (a + z) >> 1;
+              if (pc_incl[mid] > (uint32_t)e) z = mid;
+              else a = mid + 1;
+            }
+            const uint32_t before = a ? pc_incl[a - 1] : 0u;
+            const uint2 ent = src_streams[pc_src[a] + ((uint32_t)e - before)];
+            const uint32_t key = ent.y & 0xffffu, row = (ent.y >> 20) & 31u;
+            stream[stream_n + e] = uint2{ent.x, (pc_row[a] + row) | ((key - (uint32_t)wave_row0) << 20)};
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+        stream_n += batch;
+        cursor += m;
+        if (m < 64) break;  // the next piece does not fit, or there is none
+      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+
+      // ---- the wave's stream -> per-key lists in its share of LDS (a counting sort by key) ---------------------------
+      if (lane < 32) row_cnt[lane] = 0u;
+      {
+        constexpr int kPer = (SG::kListCap + 63) / 64;
+        uint2 ent[kPer];
+        uint32_t pos[kPer];
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = j * 64 + lane;
+          ent[j] = uint2{0u, 0u};
+          if (e < stream_n) ent[j] = stream[e];
+        }
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = j * 64 + lane;
+          pos[j] = 0u;
+          if (e < stream_n) pos[j] = atomicAdd(&row_cnt[(ent[j].y >> 20) & 31u], 1u);
+        }
+        {
+          const int c = lane < 32 ? (int)row_cnt[lane] : 0;
+          const int incl = wave_scan_i(c);
+          if (lane < 32) row_start[lane] = (uint32_t)(incl - c);
+          if (lane == 31) row_start[32] = (uint32_t)incl;
+        }
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = j * 64 + lane;
+          if (e < stream_n) {
+            const uint32_t at = row_start[(ent[j].y >> 20) & 31u] + pos[j];
+            lval[at] = __builtin_bit_cast(float, ent[j].x);
+            lkey[at] = (uint16_t)(ent[j].y & 0xffffu);
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+
+      // ---- per key: its list holds the queries (of this head) in whose support it lies, with score minus threshold.
+      // A group of D / 8 lanes per key, each lane 8 columns of v_j; per member it fetches its 16 bytes of dO_i and q_i and
+      // the row's delta_i and 1 / sum p (written by the dQ kernels), forms dP_ij = dO_i . v_j across the group and adds
+      // p_ij / sum p * dO_i to dV_j and u_ij (dP_ij - delta_i) * q_i to dK_j. -------------------------------------------
+      {
+        constexpr int kLPR = D / 8;         // lanes per key
+        constexpr int kGroups = 64 / kLPR;  // keys in progress per wave
+        constexpr int kDepth = 4;
+        const int grp = lane / kLPR, col = lane % kLPR;
+        const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
+        const unsigned char* qrows = reinterpret_cast<const unsigned char*>(p.q) + qo_base * 2 + col * 16;
+        const unsigned char* dorows = reinterpret_cast<const unsigned char*>(p.dout) + qo_base * 2 + col * 16;
+        const float* const delta_rows = p.delta + (size_t)(b * p.Hq + h) * N;
+        const float* const zinv_rows = p.zinv + (size_t)(b * p.Hq + h) * N;
+        for (int r0 = 0; r0 < 32; r0 += kGroups) {
+          const int r = r0 + grp;
+          const int key = wave_row0 + r;
+          const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
+          u32x4 vj = {0u, 0u, 0u, 0u};  // the lane's eight columns of v_j
+          if (key < L) vj = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
+          float acc_v[8], acc_k[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            acc_v[i] = 0.f;
+            acc_k[i] = 0.f;
+          }
+          for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+            u32x4 dd[kDepth], qq[kDepth];
+            float val[kDepth], dl[kDepth], zi[kDepth];
+#pragma unroll
+            for (int j = 0; j < kDepth; ++j) {
+              val[j] = 0.f;
+              dl[j] = 0.f;
+              zi[j] = 0.f;
+              dd[j] = u32x4{0u, 0u, 0u, 0u};
+              qq[j] = u32x4{0u, 0u, 0u, 0u};
+              if (eb + j < e_hi) {
+                const uint32_t qidx = lkey[eb + j];
+                val[j] = lval[eb + j];
+                dd[j] = *reinterpret_cast<const u32x4*>(dorows + (size_t)qidx * (D * 2));
+                qq[j] = *reinterpret_cast<const u32x4*>(qrows + (size_t)qidx * (D * 2));
+                dl[j] = delta_rows[qidx];
+                zi[j] = zinv_rows[qidx];
+              }
+            }
+            static_assert(kDepth == 4, "dot8x4 takes four members");
+            float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
+            dot8x4<T>(part, vj, dd);
+#pragma unroll
+            for (int j = 0; j < kDepth; ++j) {
+              float dof[8];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                dof[2 * i] = unpack_lo<T>(dd[j][i]);
+                dof[2 * i + 1] = unpack_hi<T>(dd[j][i]);
+              }
+              const float dp = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
+              float pr, u;
+              bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
+              const float ph = pr * zi[j], dx = u * (dp - dl[j]);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                acc_v[2 * i] = fmaf(ph, dof[2 * i], acc_v[2 * i]);
+                acc_v[2 * i + 1] = fmaf(ph, dof[2 * i + 1], acc_v[2 * i + 1]);
+                acc_k[2 * i] = fmaf(dx, unpack_lo<T>(qq[j][i]), acc_k[2 * i]);
+                acc_k[2 * i + 1] = fmaf(dx, unpack_hi<T>(qq[j][i]), acc_k[2 * i + 1]);
+              }
+            }
+          }
+          if (key < N) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc_k[i] *= p.sm_scale;
+            // fp32 partial rows of this query head (dkdv_reduce_kernel adds up the heads of a K/V head); a later part
+            // adds to what the earlier ones stored
+            float* o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
+            float* o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+            if (seg > 0) {
+              const f32x4 k0 = *reinterpret_cast<const f32x4*>(o0), k1 = *reinterpret_cast<const f32x4*>(o0 + 4);
+              const f32x4 v0 = *reinterpret_cast<const f32x4*>(o1), v1 = *reinterpret_cast<const f32x4*>(o1 + 4);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                acc_k[i] += k0[i];
+                acc_k[4 + i] += k1[i];
+                acc_v[i] += v0[i];
+                acc_v[4 + i] += v1[i];
+              }
+            }
+            *reinterpret_cast<f32x4*>(o0) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
+            *reinterpret_cast<f32x4*>(o0 + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
+            *reinterpret_cast<f32x4*>(o1) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
+            *reinterpret_cast<f32x4*>(o1 + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+          }
+        }
+      }
+      if (cursor >= n_pairs) break;
+      // (the partial rows just written are read back by the next part: by the same lanes, in program order)
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
+
+// Workgroups to launch: as many as fit the device at once (each owns one stream slot), at most `max_slots`.
+template <typename T, int D, int AM, int kKind> static int launch_attn_bwd_sparse_one(const AttnBwdParams& p, int max_slots, hipStream_t s) {
+  using SG = SparseGeo<T, D>;
+  auto kern = kKind == 2 ? attn_bwd_dkdv_stream_kernel<T, D, AM> : (kKind == 1 ? attn_bwd_dkdv_sparse_kernel<T, D, AM> : attn_bwd_dq_sparse_kernel<T, D, AM>);
   static int per_cu = 0, n_cu = 0;  // (one device family per process: gfx950; one pair per instantiation)
   if (per_cu == 0) {
     int dev = 0, blocks = 0;
@@ -1081,10 +1419,15 @@ template <typename T, int D, int AM, bool kKeys> static int launch_attn_bwd_spar
   return 0;
 }
 
-// keys = 0: the dQ kernel, 1: the dK/dV kernel
+// keys = 0: the dQ kernel, 1: the dK/dV kernel that walks for itself, 2: the dK/dV kernel that takes the dQ kernel's streams
+template <typename T, int D, int AM> static int launch_attn_bwd_sparse_am(const AttnBwdParams& p, int keys, int max_slots, hipStream_t s) {
+  if (keys == 2) return launch_attn_bwd_sparse_one<T, D, AM, 2>(p, max_slots, s);
+  if (keys == 1) return launch_attn_bwd_sparse_one<T, D, AM, 1>(p, max_slots, s);
+  return launch_attn_bwd_sparse_one<T, D, AM, 0>(p, max_slots, s);
+}
 template <typename T, int D> static int launch_attn_bwd_sparse(const AttnBwdParams& p, int am, int keys, int max_slots, hipStream_t s) {
-  if (am == ATT_15) return keys ? launch_attn_bwd_sparse_one<T, D, ATT_15, true>(p, max_slots, s) : launch_attn_bwd_sparse_one<T, D, ATT_15, false>(p, max_slots, s);
-  if (am == ATT_2) return keys ? launch_attn_bwd_sparse_one<T, D, ATT_2, true>(p, max_slots, s) : launch_attn_bwd_sparse_one<T, D, ATT_2, false>(p, max_slots, s);
+  if (am == ATT_15) return launch_attn_bwd_sparse_am<T, D, ATT_15>(p, keys, max_slots, s);
+  if (am == ATT_2) return launch_attn_bwd_sparse_am<T, D, ATT_2>(p, keys, max_slots, s);
   return 2;
 }
 

@@ -179,3 +179,31 @@ def test_sparsemax_gradients_on_flat_scores(sparse, B, H, N, D, dtype, qscale, l
             os.environ.pop("ADSP_SPARSE", None)
         else:
             os.environ["ADSP_SPARSE"] = old
+
+
+@pytest.mark.parametrize("alpha,causal,B,Hq,Hkv,N,D,dtype,lens,version,scale", [
+    (1.5, True, 2, 4, 2, 1024, 128, torch.bfloat16, [1024, 700], 2, 1.0),
+    (1.5, True, 1, 2, 1, 3000, 64, torch.float16, [2777], 2, 1.0),
+    (2.0, False, 2, 2, 2, 640, 64, torch.bfloat16, [640, 333], 1, 1.0),
+    (1.5, True, 1, 4, 4, 2048, 128, torch.bfloat16, None, 1, 0.55),  # rows with long supports: some row blocks go to the dense kernels
+])
+def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B, Hq, Hkv, N, D, dtype, lens, version, scale):
+    """The sparse-support dK/dV kernel takes the supports from the streams the dQ kernel left (default) or finds them
+    with a score walk of its own (ADSP_BWD_STREAMS=0).  Both must meet the oracle, and they must agree with each other
+    far inside the tolerance: the same members with scores that differ by a rounding at most."""
+    import os
+    varlen = None if lens is None else torch.tensor(lens, dtype=torch.int32)
+    old = os.environ.get("ADSP_BWD_STREAMS")
+    got = {}
+    try:
+        for mode in ("1", "0"):
+            os.environ["ADSP_BWD_STREAMS"] = mode
+            got[mode], want = run_case(alpha, causal, B, Hq, Hkv, N, D, dtype, varlen=varlen, version=version, seed=5, scale=scale)
+            check(got[mode], want, dtype)
+    finally:
+        if old is None:
+            os.environ.pop("ADSP_BWD_STREAMS", None)
+        else:
+            os.environ["ADSP_BWD_STREAMS"] = old
+    for a, b in zip(got["1"], got["0"]):
+        assert max_err(a, b.float().cpu(), report=False) < 1.6e-2  # (a unit in the last place of a bf16 value in [1, 2) is 7.8e-3)
