@@ -1094,8 +1094,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 // key into lists in LDS, and per key the sums over its queries.  A wave that has more members than its lists hold works
 // them off in parts; the waves of a workgroup share nothing and do not wait for each other.  A key block one of whose
 // row blocks the dQ kernel gave up (no stream) is flagged for attn_bwd_dkdv_kernel with all its heads.
+// (three waves per SIMD: the two sets of member rows in flight want 168 registers; with four waves and one set the
+// kernel was 2 % slower, with four waves and two sets it spilled)
 template <typename T, int D, int AM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE_WAVES, ADSP_SPARSE_WAVES))) void attn_bwd_dkdv_stream_kernel(AttnBwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_bwd_dkdv_stream_kernel(AttnBwdParams p) {
   using G = TileGeo<T, D>;
   using SG = SparseGeo<T, D>;
   static_assert(G::k16, "16-bit element types only");
@@ -1151,8 +1153,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     if (logical < 0) break;
 
     // ---- item -> (batch, kv head, key block, head in group), in the order of the dQ kernel's row blocks ---------
-    const int hg = logical % group;
-    const int mblk = (logical / group) % n_mblk;  // key block: with a causal mask the first ones see the most queries
+    // query head after query head, and per head key block after key block (with a causal mask the first ones see the
+    // most queries): the key blocks in flight on an XCD then gather rows of q and dO of one or two heads, some of
+    // which stay in its L2
+    const int mblk = logical % n_mblk;
+    const int hg = (logical / n_mblk) % group;
     int bkv = logical / (group * n_mblk);
     {
       const int units = p.B * p.Hkv;
@@ -1295,6 +1300,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
+      // The keys are served four at a time (a group of lanes each) and a round lasts as long as its longest list: keys
+      // in the order of their list lengths, longest first, keep the four of a round alike.  row_cnt becomes that order.
+      {
+        int rank = 0;
+        const int mine = lane < 32 ? (int)(row_start[lane + 1] - row_start[lane]) : 0;
+        for (int o = 0; o < 32; ++o) {
+          const int c = (int)(row_start[o + 1] - row_start[o]);
+          rank += (c > mine || (c == mine && o < lane)) ? 1 : 0;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane < 32) row_cnt[rank] = (uint32_t)lane;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
 
       // ---- per key: its list holds the queries (of this head) in whose support it lies, with score minus threshold.
       // A group of D / 8 lanes per key, each lane 8 columns of v_j; per member it fetches its 16 bytes of dO_i and q_i and
@@ -1305,63 +1324,86 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         constexpr int kGroups = 64 / kLPR;  // keys in progress per wave
         constexpr int kDepth = 4;
         const int grp = lane / kLPR, col = lane % kLPR;
-        const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
-        const unsigned char* qrows = reinterpret_cast<const unsigned char*>(p.q) + qo_base * 2 + col * 16;
-        const unsigned char* dorows = reinterpret_cast<const unsigned char*>(p.dout) + qo_base * 2 + col * 16;
-        const float* const delta_rows = p.delta + (size_t)(b * p.Hq + h) * N;
-        const float* const zinv_rows = p.zinv + (size_t)(b * p.Hq + h) * N;
+        const unsigned char* const vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2;
+        const unsigned char* const qrows = reinterpret_cast<const unsigned char*>(p.q) + qo_base * 2;
+        const unsigned char* const dorows = reinterpret_cast<const unsigned char*>(p.dout) + qo_base * 2;
+        const unsigned char* const delta_rows = reinterpret_cast<const unsigned char*>(p.delta + (size_t)(b * p.Hq + h) * N);
+        const unsigned char* const zinv_rows = reinterpret_cast<const unsigned char*>(p.zinv + (size_t)(b * p.Hq + h) * N);
+        const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
         for (int r0 = 0; r0 < 32; r0 += kGroups) {
-          const int r = r0 + grp;
+          const int r = (int)row_cnt[r0 + grp];
           const int key = wave_row0 + r;
           const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
           u32x4 vj = {0u, 0u, 0u, 0u};  // the lane's eight columns of v_j
-          if (key < L) vj = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
+          if (key < L) vj = *reinterpret_cast<const u32x4*>(vrows + ((uint32_t)key * (uint32_t)(D * 2) + col16));
+          // a slot without a member takes the rows of a valid query with a zero score: no weight, and no branch
+          const uint32_t safe_q = (uint32_t)(key < L ? key : L - 1);
           float acc_v[8], acc_k[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             acc_v[i] = 0.f;
             acc_k[i] = 0.f;
           }
-          for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+          // Two sets of registers: the rows of the next four members are under way while the sums of the current four are
+          // formed (a wave that waited for its loads before every round left the vector pipe idle a quarter of the time).
+          struct Quad {
             u32x4 dd[kDepth], qq[kDepth];
             float val[kDepth], dl[kDepth], zi[kDepth];
+          };
+          auto fetch = [&](Quad& m, int eb) {
 #pragma unroll
             for (int j = 0; j < kDepth; ++j) {
-              val[j] = 0.f;
-              dl[j] = 0.f;
-              zi[j] = 0.f;
-              dd[j] = u32x4{0u, 0u, 0u, 0u};
-              qq[j] = u32x4{0u, 0u, 0u, 0u};
-              if (eb + j < e_hi) {
-                const uint32_t qidx = lkey[eb + j];
-                val[j] = lval[eb + j];
-                dd[j] = *reinterpret_cast<const u32x4*>(dorows + (size_t)qidx * (D * 2));
-                qq[j] = *reinterpret_cast<const u32x4*>(qrows + (size_t)qidx * (D * 2));
-                dl[j] = delta_rows[qidx];
-                zi[j] = zinv_rows[qidx];
-              }
+              const bool has = eb + j < e_hi;
+              const uint32_t qidx = has ? (uint32_t)lkey[eb + j] : safe_q;  // (the list arrays end well inside the wave's LDS)
+              m.val[j] = has ? lval[eb + j] : 0.f;
+              const uint32_t roff = qidx * (uint32_t)(D * 2) + col16;
+              m.dd[j] = *reinterpret_cast<const u32x4*>(dorows + roff);
+              m.qq[j] = *reinterpret_cast<const u32x4*>(qrows + roff);
+              m.dl[j] = *reinterpret_cast<const float*>(delta_rows + qidx * 4u);
+              m.zi[j] = *reinterpret_cast<const float*>(zinv_rows + qidx * 4u);
             }
+          };
+          auto consume = [&](const Quad& m) {
             static_assert(kDepth == 4, "dot8x4 takes four members");
             float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
-            dot8x4<T>(part, vj, dd);
+            dot8x4<T>(part, vj, m.dd);
 #pragma unroll
             for (int j = 0; j < kDepth; ++j) {
               float dof[8];
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
-                dof[2 * i] = unpack_lo<T>(dd[j][i]);
-                dof[2 * i + 1] = unpack_hi<T>(dd[j][i]);
+                dof[2 * i] = unpack_lo<T>(m.dd[j][i]);
+                dof[2 * i + 1] = unpack_hi<T>(m.dd[j][i]);
               }
               const float dp = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
               float pr, u;
-              bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
-              const float ph = pr * zi[j], dx = u * (dp - dl[j]);
+              bwd_prob<AM>(m.val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
+              const float ph = pr * m.zi[j], dx = u * (dp - m.dl[j]);
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 acc_v[2 * i] = fmaf(ph, dof[2 * i], acc_v[2 * i]);
                 acc_v[2 * i + 1] = fmaf(ph, dof[2 * i + 1], acc_v[2 * i + 1]);
-                acc_k[2 * i] = fmaf(dx, unpack_lo<T>(qq[j][i]), acc_k[2 * i]);
-                acc_k[2 * i + 1] = fmaf(dx, unpack_hi<T>(qq[j][i]), acc_k[2 * i + 1]);
+                acc_k[2 * i] = fmaf(dx, unpack_lo<T>(m.qq[j][i]), acc_k[2 * i]);
+                acc_k[2 * i + 1] = fmaf(dx, unpack_hi<T>(m.qq[j][i]), acc_k[2 * i + 1]);
+              }
+            }
+          };
+          {
+            Quad m0, m1;
+            int eb = e_lo;
+            if (__builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull) {
+              fetch(m0, eb);
+              for (;;) {
+                eb += kDepth;
+                const bool more1 = __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull;
+                if (more1) fetch(m1, eb);
+                consume(m0);
+                if (!more1) break;
+                eb += kDepth;
+                const bool more0 = __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull;
+                if (more0) fetch(m0, eb);
+                consume(m1);
+                if (!more0) break;
               }
             }
           }
@@ -1391,7 +1433,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
       if (cursor >= n_pairs) break;
-      // (the partial rows just written are read back by the next part: by the same lanes, in program order)
+      // (the partial rows just written are read back by the next part, by this wave: the wait for its stores at the end
+      // of the next copy comes before those reads)
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
