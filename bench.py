@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
 MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.510e9, "c3": 0.5076e9, "c5": 0.595e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5371e9,
                               "c2_bwd_f32": 1.0847e9, "c2_bwd_bf16": 0.5476e9,
-                              "c4_bwd": 23.3e9}  # c4_bwd: sparse dq kernel 2.41e9 + sparse dk/dv kernel 19.21e9 + reduction 1.72e9
+                              "c4_bwd": 16.6e9}  # c4_bwd: sparse dq kernel 2.50e9 + dk/dv kernel on its streams 12.39e9 + reduction 1.72e9
 
 
 # The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
@@ -331,7 +331,7 @@ def main():
                      "roofline": {"bound": "mfma", "achieved": res["eff_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                                   "unit": "TFLOP/s", "frac": res["frac_mfma_peak"],
                                   "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
-                                  "kernel": ("attn_bwd_dq_sparse_kernel + attn_bwd_dkdv_sparse_kernel + dkdv_reduce_kernel" if args.workload == "c4_bwd" else "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel") if bwd else FWD_KERNELS[args.workload],
+                                  "kernel": ("attn_bwd_dq_sparse_kernel + attn_bwd_dkdv_stream_kernel + dkdv_reduce_kernel" if args.workload == "c4_bwd" else "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel") if bwd else FWD_KERNELS[args.workload],
                                   "flops_per_launch": res["flops_per_step"]},
                      "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k == "wall_ms_per_step"}})
         if "tiles" in res:
