@@ -15,9 +15,18 @@ def _varlen_bits(varlen):
     raise AssertionError(f"varlen must be int32/int64; got {varlen.dtype}.")
 
 
-def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_counts=None):
+def keep_supports_enabled():
+    """``ADSP_KEEP_SUPPORTS=0`` in the environment: the forward keeps nothing for the backward (comparisons, tests, or to
+    save the memory: 51 KB per 128 query rows and head)."""
+    import os
+    return os.environ.get("ADSP_KEEP_SUPPORTS", "1") != "0"
+
+
+def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_counts=None, keep_supports=False):
     """Allocate out / taus / bmask / workspace with torch and enqueue the fused forward on the
-    current stream.  Returns ``(out, taus, bmask)``."""
+    current stream.  Returns ``(out, taus, bmask)``, and with ``keep_supports`` a fourth value: the buffer in which the
+    forward keeps the supports it found for ``launch_backward`` (``None`` where the library keeps none: fp32, head dims
+    other than 64 / 128, a caller that asks for the tile statistics)."""
     _lib.require_device(q, k, v, varlen)
     lib = _lib.load()
     B, Hq, N, D = q.shape
@@ -30,9 +39,25 @@ def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_co
     ws_bytes = lib.adsp_attn_workspace_bytes(B, Hq, Hkv, N, D, dt)
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
     bits = _varlen_bits(varlen)
+    sup = None
+    if keep_supports and tile_counts is None and keep_supports_enabled():
+        sup_bytes = lib.adsp_attn_supports_bytes(B, Hq, Hkv, N, D, dt)
+        if sup_bytes:
+            sup = torch.empty((sup_bytes,), device=q.device, dtype=torch.uint8)
     with _lib.device_guard(q.device):
         stream = _lib.current_stream(q.device)
-        if version == 2:
+        if sup is not None and version == 2:
+            st = lib.adsp_attn_v2_fwd_keep(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), taus.data_ptr(),
+                                           bmask.data_ptr(), _lib.ptr(varlen), bits, B, Hq, Hkv, N, D, dt, int(niter),
+                                           _lib.ptr(ws), ws_bytes, sup.data_ptr(), sup.numel(), stream)
+            _lib.check(st, "adsp_attn_v2_fwd_keep")
+        elif sup is not None:
+            st = lib.adsp_attn_v1_fwd_keep(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), taus.data_ptr(),
+                                           bmask.data_ptr(), _lib.ptr(varlen), bits, B, Hq, N, D, dt, float(alpha),
+                                           int(bool(is_causal)), int(niter), _lib.ptr(ws), ws_bytes, sup.data_ptr(),
+                                           sup.numel(), stream)
+            _lib.check(st, "adsp_attn_v1_fwd_keep")
+        elif version == 2:
             st = lib.adsp_attn_v2_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), taus.data_ptr(),
                                       bmask.data_ptr(), _lib.ptr(varlen), bits, B, Hq, Hkv, N, D, dt, int(niter),
                                       _lib.ptr(ws), ws_bytes, stream)
@@ -43,6 +68,8 @@ def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_co
                                       int(bool(is_causal)), int(niter), _lib.ptr(ws), ws_bytes,
                                       _lib.ptr(tile_counts), stream)
             _lib.check(st, "adsp_attn_v1_fwd")
+    if keep_supports:
+        return out, taus, bmask, sup
     return out, taus, bmask
 
 
@@ -50,10 +77,11 @@ def assert_contiguous(*inputs, msg="Inputs are not contiguous."):
     assert all(t.is_contiguous() for t in inputs), msg
 
 
-def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
+def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen, supports=None):
     """Enqueue the dQ and dK/dV kernels on the current stream; returns ``(dq, dk, dv)``.
 
-    ``taus`` / ``bmask`` are the thresholds and the tile mask the forward produced.  Rows of ``dout`` past a
+    ``taus`` / ``bmask`` are the thresholds and the tile mask the forward produced, ``supports`` what it kept for this
+    call (``launch_forward(..., keep_supports=True)``) or ``None``: then the dQ kernel finds the supports again.  Rows of ``dout`` past a
     sequence's valid length are never used, whatever they hold (the kernels mask them as the reference's
     loads do, adasplash/adasplash_v2.py:1030-1033).
     """
@@ -71,9 +99,17 @@ def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen):
     ws_bytes = lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dt)
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
     with _lib.device_guard(q.device):
-        st = lib.adsp_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), taus.data_ptr(),
-                               _lib.ptr(bmask), _lib.ptr(varlen), _varlen_bits(varlen), dq.data_ptr(), dk.data_ptr(),
-                               dv.data_ptr(), delta.data_ptr(), zinv.data_ptr(), B, Hq, Hkv, N, D, dt, float(alpha),
-                               int(bool(is_causal)), _lib.ptr(ws), ws_bytes, _lib.current_stream(q.device))
-        _lib.check(st, "adsp_attn_bwd")
+        if supports is not None:
+            st = lib.adsp_attn_bwd_kept(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), taus.data_ptr(),
+                                        _lib.ptr(bmask), _lib.ptr(varlen), _varlen_bits(varlen), dq.data_ptr(),
+                                        dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), zinv.data_ptr(), B, Hq, Hkv, N, D,
+                                        dt, float(alpha), int(bool(is_causal)), _lib.ptr(ws), ws_bytes,
+                                        supports.data_ptr(), supports.numel(), _lib.current_stream(q.device))
+            _lib.check(st, "adsp_attn_bwd_kept")
+        else:
+            st = lib.adsp_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), taus.data_ptr(),
+                                   _lib.ptr(bmask), _lib.ptr(varlen), _varlen_bits(varlen), dq.data_ptr(), dk.data_ptr(),
+                                   dv.data_ptr(), delta.data_ptr(), zinv.data_ptr(), B, Hq, Hkv, N, D, dt, float(alpha),
+                                   int(bool(is_causal)), _lib.ptr(ws), ws_bytes, _lib.current_stream(q.device))
+            _lib.check(st, "adsp_attn_bwd")
     return dq, dk, dv

@@ -31,6 +31,13 @@ _SIGNATURES = {
     "adsp_attn_v2_fwd_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "adsp_attn_v1_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _dbl, _i, _i, _vp, _sz,
                               _vp, _vp]),
+    "adsp_attn_supports_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "adsp_attn_v2_fwd_keep": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _sz,
+                                   _vp]),
+    "adsp_attn_v1_fwd_keep": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _dbl, _i, _i, _vp, _sz,
+                                   _vp, _sz, _vp]),
+    "adsp_attn_bwd_kept": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
+                                _dbl, _i, _vp, _sz, _vp, _sz, _vp]),
     "adsp_attn_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "adsp_attn_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _dbl,
                            _i, _vp, _sz, _vp]),

@@ -26,10 +26,15 @@ class _SparseAttentionV1(torch.autograd.Function):
         if varlen is not None and not varlen.is_contiguous():
             varlen = varlen.contiguous()
 
-        out, taus, bmask = _attention.launch_forward(
-            q, k, v, version=1, alpha=alpha, is_causal=is_causal, niter=niter, varlen=varlen
+        # (when a gradient will be asked for, the forward keeps the supports it found: the backward then finds none again)
+        keep = any(ctx.needs_input_grad[:3])
+        res = _attention.launch_forward(
+            q, k, v, version=1, alpha=alpha, is_causal=is_causal, niter=niter, varlen=varlen,
+            keep_supports=keep,
         )
-        ctx.save_for_backward(q, k, v, taus, bmask)
+        out, taus, bmask = res[:3]
+        supports = res[3] if keep else None
+        ctx.save_for_backward(q, k, v, taus, bmask, supports)
         ctx.alpha = alpha
         ctx.is_causal = is_causal
         ctx.varlen = varlen
@@ -37,9 +42,9 @@ class _SparseAttentionV1(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, taus, bmask = ctx.saved_tensors
+        q, k, v, taus, bmask, supports = ctx.saved_tensors
         dq, dk, dv = _attention.launch_backward(
-            q, k, v, do, taus, bmask, alpha=ctx.alpha, is_causal=ctx.is_causal, varlen=ctx.varlen
+            q, k, v, do, taus, bmask, alpha=ctx.alpha, is_causal=ctx.is_causal, varlen=ctx.varlen, supports=supports
         )
         return dq, dk, dv, None, None, None, None
 

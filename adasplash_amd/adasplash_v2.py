@@ -35,18 +35,23 @@ class _SparseAttentionV2(torch.autograd.Function):
             assert varlen.is_contiguous(), "varlen must be contiguous."
         _attention.assert_contiguous(q, k, v, msg="Q, K and/or V are not contiguous.")
 
-        out, taus, bmask = _attention.launch_forward(
-            q, k, v, version=2, alpha=1.5, is_causal=True, niter=niter, varlen=varlen
+        # (when a gradient will be asked for, the forward keeps the supports it found: the backward then finds none again)
+        keep = any(ctx.needs_input_grad[:3])
+        res = _attention.launch_forward(
+            q, k, v, version=2, alpha=1.5, is_causal=True, niter=niter, varlen=varlen,
+            keep_supports=keep,
         )
-        ctx.save_for_backward(q, k, v, taus, bmask)
+        out, taus, bmask = res[:3]
+        supports = res[3] if keep else None
+        ctx.save_for_backward(q, k, v, taus, bmask, supports)
         ctx.varlen = varlen
         return out
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, taus, bmask = ctx.saved_tensors
+        q, k, v, taus, bmask, supports = ctx.saved_tensors
         dq, dk, dv = _attention.launch_backward(
-            q, k, v, do, taus, bmask, alpha=1.5, is_causal=True, varlen=ctx.varlen
+            q, k, v, do, taus, bmask, alpha=1.5, is_causal=True, varlen=ctx.varlen, supports=supports
         )
         return dq, dk, dv, None, None
 

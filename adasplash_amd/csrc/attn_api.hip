@@ -90,6 +90,8 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
   if (u == 0 && tid < 2) ctrl[64 + 2 * units + tid] = 0u;
   if (tid < 2) ctrl[64 + 2 * u + tid] = 0u;
   const int b = u / p.Hkv, kvh = u % p.Hkv, group = p.Hq / p.Hkv;
+  if (p.save_flags)  // supports kept for the backward: no row block of this K/V head has a valid stream yet
+    for (int i = tid; i < group * p.n_mblk; i += 256) p.save_flags[(size_t)(b * p.Hq + kvh * group) * p.n_mblk + i] = 0;
   int L = p.N;
   if (p.varlen) {
     long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
@@ -181,6 +183,26 @@ static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
   return w;
 }
 
+// Supports the forward keeps for the backward (adsp_attn_supports_bytes): a flag per row block, the length of every
+// (row block, wave) stream, every row's threshold minus lower bound, and the streams.
+struct SupportsLayout {
+  size_t flags_off, lens_off, tshift_off, streams_off, total;  // total = 0: nothing to keep for these dimensions
+};
+static SupportsLayout supports_layout(int B, int Hq, int Hkv, int N, int D, int dtype) {
+  SupportsLayout l = {};
+  if (dtype == ADSP_F32 || fwd_workspace(B, Hq, Hkv, N, D, dtype).slots == 0) return l;
+  const size_t items = (size_t)B * Hq * mblocks_of(N);
+  l.flags_off = 0;
+  l.lens_off = align256(items * 4);
+  l.tshift_off = align256(l.lens_off + items * 4 * 2);
+  l.streams_off = align256(l.tshift_off + (size_t)B * Hq * N * 4);
+  l.total = l.streams_off + items * kSparseSlotBytes;
+  return l;
+}
+__global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* x, long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) x[i] = 0;
+}
+
 // ADSP_SPARSE=0 in the environment keeps every row block on the dense kernel (for comparisons and tests).
 static bool sparse_enabled() {
   const char* e = getenv("ADSP_SPARSE");
@@ -197,7 +219,7 @@ static bool bwd_streams_enabled() {
 static int attn_common(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
                        const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
                        double alpha, int is_causal, int niter, int use_hist, void* workspace, size_t workspace_bytes,
-                       unsigned long long* tile_counts, hipStream_t s) {
+                       unsigned long long* tile_counts, hipStream_t s, void* supports = nullptr, size_t supports_bytes = 0) {
   if (!q || !k || !v || !out) return ADSP_ERR_NULL;
   if (dtype != ADSP_F32 && dtype != ADSP_BF16 && dtype != ADSP_F16) return ADSP_ERR_DTYPE;
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || Hq % Hkv != 0) return ADSP_ERR_SHAPE;
@@ -243,10 +265,16 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.hints = nullptr;
   p.events = nullptr;
   p.k8 = nullptr;
+  p.save_flags = nullptr;
+  p.save_lens = nullptr;
+  p.save_tshift = nullptr;
+  p.save_streams = nullptr;
 
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
     const FwdWorkspace w = fwd_workspace(B, Hq, Hkv, N, D, dtype);
+    const SupportsLayout sl = supports ? supports_layout(B, Hq, Hkv, N, D, dtype) : SupportsLayout{};
+    if (sl.total && (supports_bytes < sl.total || ((uintptr_t)supports & 15) != 0)) return ADSP_ERR_WORKSPACE;
     if (w.total && (!workspace || workspace_bytes < w.total || ((uintptr_t)workspace & 15) != 0)) return ADSP_ERR_WORKSPACE;
     unsigned char* ws = (unsigned char*)workspace;
     // Sparse-support kernel first (alpha 1.5 / 2, either entry point, no tile statistics asked for): it serves the
@@ -259,6 +287,13 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
       p.block_flags = (int32_t*)(ws + w.flags_off);
       p.events = ws + w.events_off;
       p.k8 = ws + w.k8_off;
+      if (sl.total) {
+        unsigned char* sp = (unsigned char*)supports;
+        p.save_flags = (int32_t*)(sp + sl.flags_off);
+        p.save_lens = (uint16_t*)(sp + sl.lens_off);
+        p.save_tshift = (float*)(sp + sl.tshift_off);
+        p.save_streams = sp + sl.streams_off;
+      }
       const dim3 k8_grid((unsigned)(((long long)p.Npad * (D / 16) + 255) / 256), (unsigned)(B * Hkv));
       if (dtype == ADSP_BF16) {
         hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
@@ -270,6 +305,10 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
       int rc = dtype == ADSP_BF16 ? (D == 64 ? launch_attn_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_sparse_bf16_d128(p, am, w.slots, s))
                                   : (D == 64 ? launch_attn_sparse_f16_d64(p, am, w.slots, s) : launch_attn_sparse_f16_d128(p, am, w.slots, s));
       if (rc != 0) return ADSP_ERR_LAUNCH;
+    } else if (sl.total) {  // nothing is kept by this call: the backward must not take what the buffer happens to hold
+      const long long items = (long long)B * Hq * mblocks_of(N);
+      hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((items + 255) / 256 > 1024 ? 1024 : (items + 255) / 256)), dim3(256), 0, s,
+                         (int32_t*)((unsigned char*)supports + sl.flags_off), items);
     }
   }
   // The list-carrying instance serves two and more solver steps, and a single step without the histogram (the
@@ -286,6 +325,11 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
 extern "C" size_t adsp_attn_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype) {
   if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
   return adsp::fwd_workspace(B, Hq, Hkv, N, D, dtype).total;
+}
+
+extern "C" size_t adsp_attn_supports_bytes(int B, int Hq, int Hkv, int N, int D, int dtype) {
+  if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
+  return adsp::supports_layout(B, Hq, Hkv, N, D, dtype).total;
 }
 
 extern "C" size_t adsp_attn_bmask_words(int N) {
@@ -349,6 +393,23 @@ extern "C" int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, voi
   if (alpha > 2.0) return ADSP_ERR_UNSUPPORTED;
   return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, H, H, N, D, dtype, alpha, is_causal, niter,
                            0, workspace, workspace_bytes, tile_counts, (hipStream_t)stream);
+}
+
+extern "C" int adsp_attn_v2_fwd_keep(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                                     const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
+                                     int niter, void* workspace, size_t workspace_bytes, void* supports,
+                                     size_t supports_bytes, void* stream) {
+  return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, Hq, Hkv, N, D, dtype, 1.5, 1, niter, 1,
+                           workspace, workspace_bytes, nullptr, (hipStream_t)stream, supports, supports_bytes);
+}
+
+extern "C" int adsp_attn_v1_fwd_keep(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                                     const void* varlen, int varlen_bits, int B, int H, int N, int D, int dtype,
+                                     double alpha, int is_causal, int niter, void* workspace, size_t workspace_bytes,
+                                     void* supports, size_t supports_bytes, void* stream) {
+  if (alpha > 2.0) return ADSP_ERR_UNSUPPORTED;
+  return adsp::attn_common(q, k, v, out, taus, bmask, varlen, varlen_bits, B, H, H, N, D, dtype, alpha, is_causal, niter,
+                           0, workspace, workspace_bytes, nullptr, (hipStream_t)stream, supports, supports_bytes);
 }
 
 namespace adsp {
@@ -453,10 +514,11 @@ extern "C" size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, i
   return adsp::bwd_workspace(B, Hq, Hkv, N, D, dtype).total;
 }
 
-extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* taus,
-                             const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
-                             float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
-                             int is_causal, void* workspace, size_t workspace_bytes, void* stream) {
+static int attn_bwd_impl(const void* q, const void* k, const void* v, const void* dout, const float* taus,
+                         const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
+                         float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
+                         int is_causal, void* workspace, size_t workspace_bytes, const void* supports, size_t supports_bytes,
+                         void* stream) {
   using namespace adsp;
   hipStream_t s = (hipStream_t)stream;
   if (!q || !k || !v || !dout || !taus || !dq || !dk || !dv || !delta || !zinv) return ADSP_ERR_NULL;
@@ -506,6 +568,10 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   p.streams = nullptr;
   p.stream_dir = nullptr;
   p.dir_stride = 0;
+  p.fwd_flags = nullptr;
+  p.fwd_lens = nullptr;
+  p.fwd_tshift = nullptr;
+  p.fwd_streams = nullptr;
   const int am = alpha == 1.5 ? ATT_15 : (alpha == 2.0 ? ATT_2 : ATT_GEN);
   bool sparse = false;
   BwdWorkspace w = {};
@@ -528,6 +594,17 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
         p.streams = ws + w.streams_off;
         p.stream_dir = (uint16_t*)(ws + w.dir_off);
         p.dir_stride = w.dir_stride;
+      }
+      if (supports) {  // what the forward kept: its candidate streams stand in for the dQ kernel's walk
+        const SupportsLayout sl = supports_layout(B, Hq, Hkv, N, D, dtype);
+        if (sl.total && (supports_bytes < sl.total || ((uintptr_t)supports & 15) != 0)) return ADSP_ERR_WORKSPACE;
+        if (sl.total) {
+          const unsigned char* sp = (const unsigned char*)supports;
+          p.fwd_flags = (const int32_t*)(sp + sl.flags_off);
+          p.fwd_lens = (const uint16_t*)(sp + sl.lens_off);
+          p.fwd_tshift = (const float*)(sp + sl.tshift_off);
+          p.fwd_streams = sp + sl.streams_off;
+        }
       }
       AttnParams pp = {};  // what the probe reads: q, k, lengths, dimensions, scale and the control words it clears
       pp.q = q;
@@ -597,7 +674,24 @@ extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const 
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;
 }
 
-extern "C" int adsp_version(void) { return 2; }
+extern "C" int adsp_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* taus,
+                             const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
+                             float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
+                             int is_causal, void* workspace, size_t workspace_bytes, void* stream) {
+  return attn_bwd_impl(q, k, v, dout, taus, bmask, varlen, varlen_bits, dq, dk, dv, delta, zinv, B, Hq, Hkv, N, D, dtype, alpha,
+                       is_causal, workspace, workspace_bytes, nullptr, 0, stream);
+}
+
+extern "C" int adsp_attn_bwd_kept(const void* q, const void* k, const void* v, const void* dout, const float* taus,
+                                  const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
+                                  float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
+                                  int is_causal, void* workspace, size_t workspace_bytes, const void* supports,
+                                  size_t supports_bytes, void* stream) {
+  return attn_bwd_impl(q, k, v, dout, taus, bmask, varlen, varlen_bits, dq, dk, dv, delta, zinv, B, Hq, Hkv, N, D, dtype, alpha,
+                       is_causal, workspace, workspace_bytes, supports, supports_bytes, stream);
+}
+
+extern "C" int adsp_version(void) { return 3; }
 
 #ifndef ADSP_BUILD_ID
 #define ADSP_BUILD_ID "unknown"

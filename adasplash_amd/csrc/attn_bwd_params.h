@@ -36,6 +36,12 @@ struct AttnBwdParams {
   unsigned char* streams;  // [B, Hq, n_mblk, waves, stream capacity] (score - threshold, key | row << 20) pairs
   uint16_t* stream_dir;    // [B, Hq, n_mblk, waves, dir_stride]: entry k = first stream entry with key >= 32 k
   int dir_stride;          // 4 n_mblk + 1 offsets, rounded up to an even count
+  // supports the forward kept (null: none; see AttnParams): where the flag of a row block is 1 the dQ kernel takes
+  // the forward's candidate stream and keeps the entries above the row's threshold instead of walking the scores
+  const int32_t* fwd_flags;
+  const uint16_t* fwd_lens;
+  const float* fwd_tshift;
+  const unsigned char* fwd_streams;
 };
 
 }  // namespace adsp

@@ -190,11 +190,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // ---- Q fragments; rows past the valid length are zero (their scores are never used).  The forward's threshold
     // in raw score units: the walk's accumulators start at its negative, so a positive result is a member of the
     // support ----------------------------------------------------------------------------------------------------
+    // (where the forward kept its candidate stream for this row block there is no walk: see below)
+    const bool from_fwd = p.fwd_streams != nullptr && p.fwd_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] == 1;
     const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
     uint32_t qf[G::kQRegs];
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (!from_fwd) raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + 8 * lh);
 #pragma unroll
       for (int e = 0; e < 4; ++e) qf[ks * 4 + e] = live ? raw[e] : 0u;
     }
@@ -368,6 +371,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
     };
+    if (from_fwd) {
+      // The forward's stream of this row block and wave holds every score above a lower bound of the rows' thresholds,
+      // as (score - bound, key | row) pairs in the order of its walk, and the forward left every row's threshold minus
+      // bound: the entries above it are the members, and their order stays (the table below relies on it).
+      const int n_fwd = (int)p.fwd_lens[stream_id] < SG::kListCap ? (int)p.fwd_lens[stream_id] : SG::kListCap;
+      const uint2* const src = reinterpret_cast<const uint2*>(p.fwd_streams) + stream_id * (size_t)kSparseStreamCap;
+      const float t_mine = live ? p.fwd_tshift[(size_t)(b * p.Hq + h) * N + qi] : INFINITY;  // lanes r and r + 32: row r
+      for (int e0 = 0; e0 < n_fwd; e0 += 64) {
+        const int e = e0 + lane;
+        uint2 ent = {0u, 0u};
+        if (e < n_fwd) ent = src[e];
+        const float x = __builtin_bit_cast(float, ent.x) - __shfl(t_mine, (int)((ent.y >> 20) & 31u), 64);
+        const bool keep = e < n_fwd && x > 0.f;
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(keep);
+        if (keep) {
+          const int at = stream_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+          stream[at] = uint2{__builtin_bit_cast(uint32_t, x), ent.y};
+        }
+        stream_n += __builtin_popcountll(m);
+      }
+    } else {
     walk(std::integral_constant<int, SG::kStages>{}, std::integral_constant<int, G::kKTile>{}, std::integral_constant<int, kKPer>{}, issue_k, [&](int kt, const unsigned char* kt_lds) {
       for_tile(kt, kt_lds, -lo_raw, [&](const f32x16& s0, const f32x16& s1) {
         float h00 = s0[0], h01 = s0[8], h10 = s1[0], h11 = s1[8];
@@ -385,6 +409,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       });
     });
     flush(0, nt);
+    }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
     __syncthreads();                      // every wave has left the K tiles: LDS becomes the lists
     if (s_giveup[0] | s_giveup[1]) {

@@ -41,6 +41,14 @@ struct AttnParams {
   uint32_t* hints;        // [B * Hkv + 1][2] row blocks {given up, served} per K/V head, then over all heads; zero at launch
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
   const unsigned char* k8;  // fp8 (e4m3) copy of K, [B * Hkv][Npad][D] bytes, rows past N zero: the operand of the first walk
+  // Supports kept for the backward (null: none kept).  The sparse-support kernel then writes its candidate streams to a
+  // place of their own per (row block, wave) and leaves them there, with their lengths, every row's threshold minus
+  // lower bound (raw score units: an entry is a member of the support when its value exceeds it), and a flag per row
+  // block, 1 = streams valid (the probe clears the flags; row blocks the dense kernel serves keep 0).
+  int32_t* save_flags;          // [B, Hq, n_mblk]
+  uint16_t* save_lens;          // [B, Hq, n_mblk, waves]
+  float* save_tshift;           // [B, Hq, N]
+  unsigned char* save_streams;  // [B, Hq, n_mblk, waves, stream capacity] (score - bound, key | row << 20) pairs
 };
 
 }  // namespace adsp

@@ -540,7 +540,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // row) pairs, compact and in bursts, so the tile loop rarely waits for a store.
     float* const ring = reinterpret_cast<float*>(lds_all + SG::kStages * G::kKTile + wave * SG::kRingBytes);
     uint32_t* const ring_tag = reinterpret_cast<uint32_t*>(ring + SG::kRing * 8);
-    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
+    // (kept for the backward, the stream has a place of its own per row block and wave)
+    const size_t stream_id = ((size_t)(b * p.Hq + h) * n_mblk + mblk) * NW + wave;
+    uint2* const stream = p.save_streams ? reinterpret_cast<uint2*>(p.save_streams) + stream_id * (size_t)kSparseStreamCap
+                                         : reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
     int ring_n = 0, stream_n = 0;  // wave-uniform
     // (kt: the tile being worked on; a stream that fills faster than the tiles go by will not last: give up early)
     auto flush = [&](int parity, int kt) {
@@ -723,6 +726,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         row_cnt[lq] = (uint32_t)(w - row_lo);
         row_inv[lq] = (live && psum > 0.f) ? 1.f / psum : 0.f;
         if (live && p.taus) p.taus[(size_t)(b * p.Hq + h) * N + qi] = (lo_raw + t) * qs;
+        if (live && p.save_tshift) p.save_tshift[(size_t)(b * p.Hq + h) * N + qi] = t;
       }
     }
 
@@ -772,8 +776,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     __syncthreads();  // every wave's tile marks are in
     if (bmask_out)
       for (int i = tid; i < p.mask_words; i += SG::kThreads) bmask_out[i] = (int32_t)mask_out[i];
+    if (p.save_lens && lane == 0) p.save_lens[stream_id] = (uint16_t)stream_n;
     if (tid == 0) {
       *flag = 0;
+      if (p.save_flags) p.save_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] = 1;
       if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
         atomicAdd(hint + 1, 1u);
         atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);

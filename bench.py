@@ -147,11 +147,12 @@ def bench_attention(name, steps, warmup, device, backward=False):
         from adasplash_amd import _attention
 
         assert name in ("c4", "c3")
-        out, taus, bmask = _attention.launch_forward(q, k, v, version=2, alpha=1.5, is_causal=True, niter=1,
-                                                     varlen=varlen)
+        # (as the autograd function does: the forward keeps the supports it found for the backward)
+        out, taus, bmask, supports = _attention.launch_forward(q, k, v, version=2, alpha=1.5, is_causal=True, niter=1,
+                                                               varlen=varlen, keep_supports=True)
         dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(7)).to(q.dtype).to(device)
         fn = lambda: _attention.launch_backward(q, k, v, dout, taus, bmask, alpha=1.5, is_causal=True,  # noqa: E731
-                                                varlen=varlen)
+                                                varlen=varlen, supports=supports)
         flops = 2.5 * flops
         cfg = dict(cfg, workload=cfg["workload"].replace("fwd", "bwd (dq, dk, dv)"))
     if name == "c3" and not backward:

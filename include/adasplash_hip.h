@@ -139,6 +139,34 @@ int adsp_attn_v1_fwd(const void* q, const void* k, const void* v, void* out, flo
                      unsigned long long* tile_counts, void* stream);
 
 /*
+ * Supports kept for the backward.  No counterpart in the reference (its backward recomputes the scores of every tile of
+ * the mask).  The sparse-support forward kernel finds, for every row, the few keys with a non-zero probability; the
+ * _keep variants of the two forward entry points leave what they found in `supports` -- per 128-row block of a query
+ * head its streams of (score, key) pairs, their lengths, every row's threshold relative to the streams' scores and a
+ * flag -- and adsp_attn_bwd_kept, given the same buffer untouched, takes the supports from there instead of walking
+ * the scores again.  adsp_attn_supports_bytes() is the size of that buffer (51 KiB per 128 query rows and head plus
+ * 4 bytes per row; 0 where nothing is kept: fp32, head dims other than 64 and 128, N > 65536; `supports` may then be
+ * NULL).  16-byte aligned device memory owned by the caller; it must hold what the forward wrote for the same
+ * q, k, v, varlen until the backward has run.  Row blocks the forward served with its dense kernel keep no supports
+ * and the backward walks them as adsp_attn_bwd does; with supports == NULL the three calls are adsp_attn_v2_fwd,
+ * adsp_attn_v1_fwd (without tile statistics) and adsp_attn_bwd.
+ */
+size_t adsp_attn_supports_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
+int adsp_attn_v2_fwd_keep(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                          const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
+                          int niter, void* workspace, size_t workspace_bytes, void* supports, size_t supports_bytes,
+                          void* stream);
+int adsp_attn_v1_fwd_keep(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
+                          const void* varlen, int varlen_bits, int B, int H, int N, int D, int dtype, double alpha,
+                          int is_causal, int niter, void* workspace, size_t workspace_bytes, void* supports,
+                          size_t supports_bytes, void* stream);
+int adsp_attn_bwd_kept(const void* q, const void* k, const void* v, const void* dout, const float* taus,
+                       const int32_t* bmask, const void* varlen, int varlen_bits, void* dq, void* dk, void* dv,
+                       float* delta, float* zinv, int B, int Hq, int Hkv, int N, int D, int dtype, double alpha,
+                       int is_causal, void* workspace, size_t workspace_bytes, const void* supports,
+                       size_t supports_bytes, void* stream);
+
+/*
  * Workspace of adsp_attn_bwd in bytes; 0 for fp32 and for the head dims the sparse-support kernels do not serve (then
  * `workspace` may be NULL).  For the 16-bit element types at head dims 64 and 128 (sequences of up to 65536 keys): the
  * counters, flags and candidate streams of the sparse-support backward kernels, fp32 partial rows of dk and dv per

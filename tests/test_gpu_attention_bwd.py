@@ -207,3 +207,34 @@ def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B
             os.environ["ADSP_BWD_STREAMS"] = old
     for a, b in zip(got["1"], got["0"]):
         assert max_err(a, b.float().cpu(), report=False) < 1.6e-2  # (a unit in the last place of a bf16 value in [1, 2) is 7.8e-3)
+
+
+@pytest.mark.parametrize("alpha,causal,B,Hq,Hkv,N,D,dtype,lens,version,scale,sparse", [
+    (1.5, True, 2, 4, 2, 1024, 128, torch.bfloat16, [1024, 700], 2, 1.0, "1"),
+    (1.5, True, 1, 2, 1, 3000, 64, torch.float16, [2777], 2, 1.0, "1"),
+    (2.0, False, 2, 2, 2, 640, 64, torch.bfloat16, [640, 333], 1, 1.0, "1"),
+    (1.5, True, 1, 4, 4, 2048, 128, torch.bfloat16, None, 1, 0.55, "1"),  # some row blocks go to the dense kernels: no supports kept for them
+    (1.5, True, 2, 2, 2, 512, 64, torch.bfloat16, [512, 300], 2, 1.0, "0"),   # the dense forward keeps nothing: every flag is cleared
+])
+def test_backward_with_and_without_the_supports_the_forward_kept(alpha, causal, B, Hq, Hkv, N, D, dtype, lens, version, scale, sparse):
+    """With a gradient asked for the forward keeps the supports it found and the dQ kernel takes them from there
+    (default); ADSP_KEEP_SUPPORTS=0 makes it find them again with its score walk.  Both must meet the oracle and agree
+    with each other (the same members up to scores that differ by a rounding)."""
+    import os
+    varlen = None if lens is None else torch.tensor(lens, dtype=torch.int32)
+    old = {k: os.environ.get(k) for k in ("ADSP_KEEP_SUPPORTS", "ADSP_SPARSE")}
+    got = {}
+    try:
+        os.environ["ADSP_SPARSE"] = sparse
+        for mode in ("1", "0"):
+            os.environ["ADSP_KEEP_SUPPORTS"] = mode
+            got[mode], want = run_case(alpha, causal, B, Hq, Hkv, N, D, dtype, varlen=varlen, version=version, seed=6, scale=scale)
+            check(got[mode], want, dtype)
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    for a, b in zip(got["1"], got["0"]):
+        assert max_err(a, b.float().cpu(), report=False) < 1.6e-2  # (a unit in the last place of a bf16 value in [1, 2) is 7.8e-3)
