@@ -492,8 +492,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       constexpr int kGroups = 64 / kLPR;  // rows in progress per wave
       constexpr int kDepth = 4;
       const int grp = lane / kLPR, col = lane % kLPR;
-      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
-      const unsigned char* krows = kglob + col * 16;
+      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2;
+      const unsigned char* krows = kglob;
+      const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
       const unsigned char* dorows = reinterpret_cast<const unsigned char*>(p.dout) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
       unsigned char* dqrows = reinterpret_cast<unsigned char*>(p.dq) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
       for (int r0 = 0; r0 < 32; r0 += kGroups) {
@@ -514,15 +515,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           float val[kDepth];
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
-            val[j] = 0.f;
-            vv[j] = u32x4{0u, 0u, 0u, 0u};
-            kk[j] = u32x4{0u, 0u, 0u, 0u};
-            if (eb + j < e_hi) {
-              const uint32_t key = lkey[eb + j];
-              val[j] = lval[eb + j];
-              vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
-              kk[j] = *reinterpret_cast<const u32x4*>(krows + (size_t)key * (D * 2));
-            }
+            // a slot without a member takes the first key's rows (always valid) with a zero score: no weight, no branch
+            const bool has = eb + j < e_hi;
+            const uint32_t key = has ? (uint32_t)lkey[eb + j] : 0u;  // (the list arrays end well inside the wave's LDS)
+            val[j] = has ? lval[eb + j] : 0.f;
+            const uint32_t roff = key * (uint32_t)(D * 2) + col16;
+            vv[j] = *reinterpret_cast<const u32x4*>(vrows + roff);
+            kk[j] = *reinterpret_cast<const u32x4*>(krows + roff);
           }
           static_assert(kDepth == 4, "dot8x4 takes four members");
           float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
