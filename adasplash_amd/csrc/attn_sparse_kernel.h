@@ -739,7 +739,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       constexpr int kGroups = 64 / kLPR;  // rows in progress per wave
       constexpr int kDepth = ADSP_GATHER_DEPTH;
       const int grp = lane / kLPR, col = lane % kLPR;
-      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2 + col * 16;
+      const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2;
+      const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
       unsigned char* obase = reinterpret_cast<unsigned char*>(p.out) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
       for (int r0 = 0; r0 < 32; r0 += kGroups) {
         const int r = r0 + grp;
@@ -752,13 +753,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           uint32_t pw[kDepth];
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
-            pw[j] = 0u;
-            vv[j] = u32x4{0u, 0u, 0u, 0u};
-            if (eb + j < e_hi) {
-              const uint32_t key = lkey[eb + j];
-              pw[j] = __builtin_bit_cast(uint32_t, lval[eb + j]);
-              vv[j] = *reinterpret_cast<const u32x4*>(vrows + (size_t)key * (D * 2));
-            }
+            // a slot without a member takes the first key's row (always valid) with a zero weight: no zeroing, no branch
+            const bool has = eb + j < e_hi;
+            const uint32_t key = has ? (uint32_t)lkey[eb + j] : 0u;  // (the list arrays end well inside the wave's LDS)
+            pw[j] = has ? __builtin_bit_cast(uint32_t, lval[eb + j]) : 0u;
+            vv[j] = *reinterpret_cast<const u32x4*>(vrows + (key * (uint32_t)(D * 2) + col16));
           }
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
