@@ -497,8 +497,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
       const unsigned char* dorows = reinterpret_cast<const unsigned char*>(p.dout) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
       unsigned char* dqrows = reinterpret_cast<unsigned char*>(p.dq) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
+      // The rows are served kGroups at a time and a round lasts as long as its longest list: rows in the order of their
+      // list lengths, longest first, keep the rows of a round alike.  row_cnt (free since the sort) becomes that order.
+      {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        int rank = 0;
+        const int mine = lane < 32 ? (int)(row_start[lane + 1] - row_start[lane]) : 0;
+        for (int o = 0; o < 32; ++o) {
+          const int c = (int)(row_start[o + 1] - row_start[o]);
+          rank += (c > mine || (c == mine && o < lane)) ? 1 : 0;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane < 32) row_cnt[rank] = (uint32_t)lane;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
       for (int r0 = 0; r0 < 32; r0 += kGroups) {
-        const int r = r0 + grp;
+        const int r = (int)row_cnt[r0 + grp];
         const bool row_live = wave_row0 + r < L;
         const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
         u32x4 dov = {0u, 0u, 0u, 0u};  // the lane's eight columns of dO_i (rows past the valid length may hold anything: not read)

@@ -742,8 +742,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2;
       const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
       unsigned char* obase = reinterpret_cast<unsigned char*>(p.out) + (qo_base + (size_t)wave_row0 * D) * 2 + col * 16;
+      // The rows are served kGroups at a time and a round lasts as long as its longest support: rows in the order of
+      // their supports' sizes, longest first, keep the rows of a round alike.
+      uint8_t* const order = reinterpret_cast<uint8_t*>(row_inv + 32);
+      {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        int rank = 0;
+        const int mine = lane < 32 ? (int)row_cnt[lane] : 0;
+        for (int o = 0; o < 32; ++o) {
+          const int c = (int)row_cnt[o];
+          rank += (c > mine || (c == mine && o < lane)) ? 1 : 0;
+        }
+        if (lane < 32) order[rank] = (uint8_t)lane;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
       for (int r0 = 0; r0 < 32; r0 += kGroups) {
-        const int r = r0 + grp;
+        const int r = (int)order[r0 + grp];
         const int e_lo = (int)row_start[r], e_hi = e_lo + (int)row_cnt[r];
         float acc[8];
 #pragma unroll
