@@ -660,7 +660,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
     else rc = D == 64 ? launch_attn_bwd_sparse_f16_d64(p, am, kind, w.slots, s) : launch_attn_bwd_sparse_f16_d128(p, am, kind, w.slots, s);
     if (rc != 0) return ADSP_ERR_LAUNCH;
     if (kBwdTable[dtype][head_dim_slot(D)](p, am, 2, s) != 0) return ADSP_ERR_LAUNCH;
-    if (w.part_bytes) {
+    if (w.part_bytes && !(p.streams && Hq == Hkv)) {  // (with one query head per K/V head the kernel on the streams writes dK and dV itself)
       const long long threads = (long long)B * Hkv * N * (D / 8);
       const dim3 grid((unsigned)((threads + 255) / 256));
       if (dtype == ADSP_BF16)

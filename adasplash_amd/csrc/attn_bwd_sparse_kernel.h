@@ -1132,7 +1132,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 // streams of the head that hold its keys (row blocks from its own on with a causal mask) into a stream of its own, as
 // (score - threshold, query | key << 20) pairs, and from there on does what the walking kernel does: a counting sort by
 // key into lists in LDS, and per key the sums over its queries.  A wave that has more members than its lists hold works
-// them off in parts; the waves of a workgroup share nothing and do not wait for each other.  A key block one of whose
+// them off in parts; the waves of a workgroup share nothing and do not wait for each other.  The sums are fp32 partial
+// rows per query head for dkdv_reduce_kernel; where a K/V head has a single query head the last part writes dK and dV
+// in the element type and there is no reduction.  A key block one of whose
 // row blocks the dQ kernel gave up (no stream) is flagged for attn_bwd_dkdv_kernel with all its heads.
 // (three waves per SIMD: the two sets of member rows in flight want 168 registers; with four waves and one set the
 // kernel was 2 % slower, with four waves and two sets it spilled)
@@ -1211,7 +1213,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
       L = (int)(l < 0 ? 0 : (l > N ? N : l));
     }
-    if (m0 >= L) continue;  // key block entirely inside the padding: dkdv_reduce_kernel writes its zeros
+    const bool direct = group == 1;  // a K/V head with a single query head: no sums over heads, dK and dV are written here
+    if (m0 >= L) {  // key block entirely inside the padding: zero gradient (dkdv_reduce_kernel writes it unless `direct`)
+      if (direct) {
+        constexpr int kRowDw = D * 2 / 4;
+        const size_t at = (((size_t)(b * p.Hkv + kvh) * N + m0) * D) * 2 / 4;
+        uint32_t* const k32o = reinterpret_cast<uint32_t*>(p.dk) + at;
+        uint32_t* const v32o = reinterpret_cast<uint32_t*>(p.dv) + at;
+        const int rows = (N - m0) < BM ? (N - m0) : BM;
+        for (int i = tid; i < rows * kRowDw; i += SG::kThreads) {
+          k32o[i] = 0u;
+          v32o[i] = 0u;
+        }
+      }
+      continue;
+    }
     // a key block that any query head gives up goes to attn_bwd_dkdv_kernel with all its heads
     int32_t* const flag = p.kv_flags + ((size_t)(b * p.Hkv + kvh) * n_mblk + mblk);
     const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
@@ -1468,10 +1484,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 acc_v[4 + i] += v1[i];
               }
             }
-            *reinterpret_cast<f32x4*>(o0) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
-            *reinterpret_cast<f32x4*>(o0 + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
-            *reinterpret_cast<f32x4*>(o1) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
-            *reinterpret_cast<f32x4*>(o1 + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+            if (direct && cursor >= n_pairs) {  // the last part of the only head: the sums in the element type
+              const u32x4 wk = {pack2<T>(acc_k[0], acc_k[1]), pack2<T>(acc_k[2], acc_k[3]), pack2<T>(acc_k[4], acc_k[5]), pack2<T>(acc_k[6], acc_k[7])};
+              const u32x4 wv = {pack2<T>(acc_v[0], acc_v[1]), pack2<T>(acc_v[2], acc_v[3]), pack2<T>(acc_v[4], acc_v[5]), pack2<T>(acc_v[6], acc_v[7])};
+              *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dk) + kv_base + (size_t)key * D + col * 8) = wk;
+              *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dv) + kv_base + (size_t)key * D + col * 8) = wv;
+            } else {
+              *reinterpret_cast<f32x4*>(o0) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
+              *reinterpret_cast<f32x4*>(o0 + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
+              *reinterpret_cast<f32x4*>(o1) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
+              *reinterpret_cast<f32x4*>(o1 + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+            }
           }
         }
       }
