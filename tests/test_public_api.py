@@ -171,6 +171,13 @@ def test_sizing_helpers_and_status_strings():
     assert 8 * slot < small < 8 * slot + 2 * 64 * 128 * 3 + 1024
     assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_F32) == 0
     assert lib.adsp_attn_bmask_words(8192) == 64 * 4 and lib.adsp_attn_bmask_words(64) == 1
+    # supports kept for the backward: per 128-row block of a query head a flag, four stream lengths and the four
+    # streams, plus a word per row; nothing where the sparse-support kernel does not run
+    items = 8 * 32 * 64
+    assert lib.adsp_attn_supports_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) == items * 4 + items * 8 + 8 * 32 * 8192 * 4 + items * slot
+    assert lib.adsp_attn_supports_bytes(8, 32, 8, 8192, 128, _lib.ADSP_F32) == 0
+    assert lib.adsp_attn_supports_bytes(2, 2, 2, 100, 32, _lib.ADSP_F16) == 0
+    assert lib.adsp_attn_bwd_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) > 2 * 8 * 32 * 8192 * 128 * 4 + items * slot
     assert lib.adsp_status_string(0) == b"ok"
     assert all(len(lib.adsp_status_string(s)) > 0 for s in range(0, 9))
 
