@@ -141,7 +141,17 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
     for (int it = 0; it < 14; ++it) {
       const float a = 0.5f * (lo + hi);
       const float Q = 0.5f * erfcf(a * 0.70710678f), phi = 0.39894228f * __expf(-0.5f * a * a);
-      const float f = am == ATT_2 ? n * sd * (phi - a * Q) : n * var * ((1.f + a * a) * Q - a * phi);
+      float f;
+      if (am == ATT_2) f = n * sd * (phi - a * Q);
+      else if (am == ATT_15) f = n * var * ((1.f + a * a) * Q - a * phi);
+      else {  // any alpha: n E[(sd (Z - a))_+^c0] by the midpoint rule over [a, a + 8]
+        float acc = 0.f;
+        for (int i = 0; i < 32; ++i) {
+          const float x = 0.25f * ((float)i + 0.5f);
+          acc += __expf(p.c0 * __logf(sd * x)) * 0.39894228f * __expf(-0.5f * (a + x) * (a + x));
+        }
+        f = n * acc * 0.25f;
+      }
       if (f > 1.f) lo = a;
       else hi = a;
     }
@@ -279,7 +289,8 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
     unsigned char* ws = (unsigned char*)workspace;
     // Sparse-support kernel first (alpha 1.5 / 2, either entry point, no tile statistics asked for): it serves the
     // row blocks whose supports are short and flags the others for the kernel below.
-    const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && !tile_counts &&
+    // (any other alpha in [1.125, 2) as well: below that its solver on the lists would need too many rounds)
+    const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2 || (alpha >= 1.125 && alpha < 2.0)) && !tile_counts &&
                         (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
     if (sparse) {
       p.queue = (uint32_t*)(ws + w.queue_off);
@@ -583,7 +594,8 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
     if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0)) return ADSP_ERR_WORKSPACE;
     // Sparse-support dQ kernel first (alpha 1.5 / 2): it serves the row blocks whose supports are short and flags the
     // others for attn_bwd_dq_kernel below; the dK/dV kernel reads delta and 1 / sum p from whichever of the two wrote them.
-    sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2) && (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
+    sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2 || (alpha >= 1.125 && alpha < 2.0)) &&
+             (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
     if (sparse) {
       unsigned char* ws = (unsigned char*)workspace;
       p.queue = (uint32_t*)(ws + w.queue_off);
@@ -617,6 +629,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
       pp.N = N;
       pp.causal = p.causal;
       pp.qscale = p.qscale;
+      pp.c0 = p.c0;
       pp.queue = p.queue;
       pp.hints = p.hints;
       int rc;

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   using SG = SparseGeo<T, D>;
   using KS = Swz<G::kKRow>;
   static_assert(G::k16, "16-bit element types only");
-  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  static_assert(AM == ATT_15 || AM == ATT_2 || AM == ATT_GEN, "alpha = 1.5, 2 or any other in (1, 2)");
   constexpr int NW = SG::kNW, BM = SG::kBM;
   __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
   __shared__ int s_item, s_skip;
@@ -603,7 +603,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   using SG = SparseGeo<T, D>;
   using KS = Swz<G::kKRow>;
   static_assert(G::k16, "16-bit element types only");
-  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  static_assert(AM == ATT_15 || AM == ATT_2 || AM == ATT_GEN, "alpha = 1.5, 2 or any other in (1, 2)");
   constexpr int NW = SG::kNW, BM = SG::kBM;
   __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
   __shared__ int s_item, s_skip;
@@ -1143,7 +1143,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   using G = TileGeo<T, D>;
   using SG = SparseGeo<T, D>;
   static_assert(G::k16, "16-bit element types only");
-  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  static_assert(AM == ATT_15 || AM == ATT_2 || AM == ATT_GEN, "alpha = 1.5, 2 or any other in (1, 2)");
   constexpr int NW = SG::kNW, BM = SG::kBM;
   __shared__ __align__(16) unsigned char lds_all[NW * SG::kWaveLds];
   __shared__ int s_item, s_skip;
@@ -1537,6 +1537,7 @@ template <typename T, int D, int AM> static int launch_attn_bwd_sparse_am(const 
 template <typename T, int D> static int launch_attn_bwd_sparse(const AttnBwdParams& p, int am, int keys, int max_slots, hipStream_t s) {
   if (am == ATT_15) return launch_attn_bwd_sparse_am<T, D, ATT_15>(p, keys, max_slots, s);
   if (am == ATT_2) return launch_attn_bwd_sparse_am<T, D, ATT_2>(p, keys, max_slots, s);
+  if (am == ATT_GEN) return launch_attn_bwd_sparse_am<T, D, ATT_GEN>(p, keys, max_slots, s);
   return 2;
 }
 

@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   using KS8 = Swz<SG::kK8Row>;
   static_assert(G::k16, "16-bit element types only");
   static_assert(D % 64 == 0, "the fp8 products take 64 values of the head dim at a time");
-  static_assert(AM == ATT_15 || AM == ATT_2, "alpha = 1.5 or 2");
+  static_assert(AM == ATT_15 || AM == ATT_2 || AM == ATT_GEN, "alpha = 1.5, 2 or any other in (1, 2)");
   constexpr int NW = SG::kNW, BM = SG::kBM;
   __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
   __shared__ int s_item, s_skip;
@@ -520,12 +520,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           if constexpr (AM == ATT_15) {
             a0 = fmaf(u, u, a0);
             a1 += u;
-          } else {
+          } else if constexpr (AM == ATT_2) {
             a0 += u;
             a1 += u > 0.f ? 1.f : 0.f;
+          } else {  // any alpha: sums of (qs u)^c0 and (qs u)^(c0 - 1), in z units
+            const float uz = u * qs;
+            const float pw = u > 0.f ? fast_exp2(p.c0 * fast_log2(uz)) : 0.f;
+            a0 += pw;
+            a1 += u > 0.f ? pw * fast_rcp(uz) : 0.f;
           }
         }
-        const float step = (AM == ATT_15) ? (a0 - target) / (2.f * a1) : (a0 - target) / a1;
+        // (any alpha: f = a0 - 1, f' = -c0 qs a1 per raw unit; the steps of a convex decreasing f from the left never
+        // pass its root, converged or not: what the eight rounds leave is a valid bound)
+        const float step = (AM == ATT_15) ? (a0 - target) / (2.f * a1) : (AM == ATT_2) ? (a0 - target) / a1 : (a0 - 1.f) * inv_qs / (p.c0 * a1);
         t += (a1 > 0.f && step > 0.f) ? step : 0.f;
       }
       // the margin covers the rounding of the iteration; rows past the valid length take no part in walk 2
@@ -686,22 +693,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     float t = 0.f;  // threshold minus lo, raw units
     {
       const float target = (AM == ATT_15) ? inv_qs * inv_qs : inv_qs;
-      for (int it = 0; it < 24; ++it) {
+      // (any alpha: the steps shrink like 1 - 1 / c0 while f is large, so the rounds are more; the launch keeps alphas
+      // whose c0 = 1 / (alpha - 1) exceeds 8 on the dense kernel)
+      for (int it = 0; it < (AM == ATT_GEN ? 96 : 24); ++it) {
         float a0 = 0.f, a1 = 0.f;
         for (int e = row_lo + lh; e < row_end; e += 2) {
           const float u = fmaxf(lval[e] - t, 0.f);
           if constexpr (AM == ATT_15) {
             a0 = fmaf(u, u, a0);
             a1 += u;
-          } else {
+          } else if constexpr (AM == ATT_2) {
             a0 += u;
             a1 += u > 0.f ? 1.f : 0.f;
+          } else {
+            const float uz = u * qs;
+            const float pw = u > 0.f ? fast_exp2(p.c0 * fast_log2(uz)) : 0.f;
+            a0 += pw;
+            a1 += u > 0.f ? pw * fast_rcp(uz) : 0.f;
           }
         }
         a0 += __shfl_xor(a0, 32, 64);
         a1 += __shfl_xor(a1, 32, 64);
-        const float step = (AM == ATT_15) ? (a0 - target) / (2.f * a1) : (a0 - target) / a1;
-        const bool move = a1 > 0.f && step > 1e-7f * inv_qs;
+        const float step = (AM == ATT_15) ? (a0 - target) / (2.f * a1) : (AM == ATT_2) ? (a0 - target) / a1 : (a0 - 1.f) * inv_qs / (p.c0 * a1);
+        const bool move = a1 > 0.f && step > (AM == ATT_GEN ? 2e-6f : 1e-7f) * inv_qs;  // (any alpha: the powers carry a relative 1e-6)
         t += move ? step : 0.f;
         if (__builtin_amdgcn_ballot_w64(move) == 0ull) break;
       }
@@ -716,7 +730,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           const float u = lval[e] - t;
           const uint16_t key = lkey[e];
           if (u > 0.f) {
-            const float pv = (AM == ATT_15) ? u * u : u;
+            const float pv = (AM == ATT_15) ? u * u : (AM == ATT_2) ? u : fast_exp2(p.c0 * fast_log2(u * qs));
             lval[w] = __builtin_bit_cast(float, pack2<T>(pv, 0.f));  // the pair (p, 0) of the element type, as the output loop takes it
             lkey[w] = key;
             ++w;
@@ -829,6 +843,7 @@ template <typename T, int D, int AM> static int launch_attn_sparse_one(const Att
 template <typename T, int D> static int launch_attn_sparse(const AttnParams& p, int am, int max_slots, hipStream_t s) {
   if (am == ATT_15) return launch_attn_sparse_one<T, D, ATT_15>(p, max_slots, s);
   if (am == ATT_2) return launch_attn_sparse_one<T, D, ATT_2>(p, max_slots, s);
+  if (am == ATT_GEN) return launch_attn_sparse_one<T, D, ATT_GEN>(p, max_slots, s);
   return 2;
 }
 

@@ -215,6 +215,8 @@ def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B
     (2.0, False, 2, 2, 2, 640, 64, torch.bfloat16, [640, 333], 1, 1.0, "1"),
     (1.5, True, 1, 4, 4, 2048, 128, torch.bfloat16, None, 1, 0.55, "1"),  # some row blocks go to the dense kernels: no supports kept for them
     (1.5, True, 2, 2, 2, 512, 64, torch.bfloat16, [512, 300], 2, 1.0, "0"),   # the dense forward keeps nothing: every flag is cleared
+    (1.333, False, 1, 2, 2, 1500, 128, torch.bfloat16, [1400], 1, 1.5, "1"),  # any alpha in [1.125, 2) takes the same kernels
+    (1.8, True, 2, 2, 2, 768, 64, torch.float16, [768, 500], 1, 1.5, "1"),
 ])
 def test_backward_with_and_without_the_supports_the_forward_kept(alpha, causal, B, Hq, Hkv, N, D, dtype, lens, version, scale, sparse):
     """With a gradient asked for the forward keeps the supports it found and the dQ kernel takes them from there
