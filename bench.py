@@ -35,9 +35,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these
 # same workloads, each counter scaled by what it reads for a plain 1 GiB copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
-MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.471e9, "c3": 0.5064e9, "c5": 0.599e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5371e9,
+MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.467e9, "c3": 0.5079e9, "c5": 0.577e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5371e9,
                               "c2_bwd_f32": 1.0847e9, "c2_bwd_bf16": 0.5476e9,
-                              "c4_bwd": 15.4e9}  # c4_bwd: sparse dq kernel 2.33e9 + dk/dv kernel on its streams 11.38e9 + reduction 1.72e9
+                              "c4_bwd": 15.4e9}  # c4_bwd: sparse dq kernel 2.33e9 + dk/dv kernel on its streams 11.40e9 + reduction 1.72e9
 
 
 # The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
@@ -46,7 +46,7 @@ MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.471e9, "c3": 0.5064e9, "c5": 0.599e9, "c2_
 # copy of K and the sparse-support kernel step aside and the dense kernel does all the work).
 FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + fp8 copy of K + this + attn_fwd_kernel on leftovers)",
                "c3": "attn_fwd_kernel<bf16, 64, single step> (step = probe + sparse-support kernel stepping aside + this)",
-               "c5": "attn_fwd_kernel<bf16, 64, generic alpha, candidate lists>"}
+               "c5": "attn_fwd_sparse_kernel<bf16, 64, generic alpha> (step = probe + fp8 copy of K + this + attn_fwd_kernel on leftovers)"}
 
 
 def _events_ms(fn, steps, warmup):
