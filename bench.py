@@ -11,7 +11,7 @@ Workloads (``--workload``):
   c5   adasplash_v1 non-causal alpha=1.333 niter=10, B=2 H=16 N=16384 D=64 bf16, q,k x3
   c2   entmax rows x[16384, 8192] = 4*N(0,1), bf16 and fp32, alpha in {1.5, 2}
   c2_bwd  entmax rows backward on the same shape (reads y, writes dx, reads dy on the support only)
-  c4_bwd, c3_bwd   dq, dk, dv of the c4 / c3 forward (2.5 x its dense-equivalent FLOPs per step)
+  c4_bwd, c3_bwd, c5_bwd   dq, dk, dv of the c4 / c3 / c5 forward (2.5 x its dense-equivalent FLOPs per step)
 The default run also times c3, c5, the entmax rows workloads (c2, c2_bwd) and the c4 backward and reports them under
 ``extra``, with the v2 tile statistics of the headline workload (key tiles of 128 rows x 64 keys inside the causal /
 valid domain, those the block mask keeps, and the share of row blocks the sparse-support kernel served).
@@ -37,7 +37,8 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
 MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.467e9, "c3": 0.5079e9, "c5": 0.577e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5371e9,
                               "c2_bwd_f32": 1.0847e9, "c2_bwd_bf16": 0.5476e9,
-                              "c4_bwd": 15.4e9}  # c4_bwd: sparse dq kernel 2.33e9 + dk/dv kernel on its streams 11.40e9 + reduction 1.72e9
+                              "c4_bwd": 15.4e9,
+                              "c5_bwd": 0.962e9}  # c4_bwd: sparse dq kernel 2.33e9 + dk/dv kernel on its streams 11.40e9 + reduction 1.72e9
 
 
 # The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
@@ -47,6 +48,9 @@ MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.467e9, "c3": 0.5079e9, "c5": 0.577e9, "c2_
 FWD_KERNELS = {"c4": "attn_fwd_sparse_kernel<bf16, 128> (step = probe + fp8 copy of K + this + attn_fwd_kernel on leftovers)",
                "c3": "attn_fwd_kernel<bf16, 64, single step> (step = probe + sparse-support kernel stepping aside + this)",
                "c5": "attn_fwd_sparse_kernel<bf16, 64, generic alpha> (step = probe + fp8 copy of K + this + attn_fwd_kernel on leftovers)"}
+_BWD_SPARSE = "attn_bwd_dq_sparse_kernel + attn_bwd_dkdv_stream_kernel"
+BWD_KERNELS = {"c4_bwd": _BWD_SPARSE + " + dkdv_reduce_kernel", "c3_bwd": "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel",
+               "c5_bwd": _BWD_SPARSE + " (generic alpha; one query head per K/V head: no reduction)"}
 
 
 def _events_ms(fn, steps, warmup):
@@ -146,17 +150,21 @@ def bench_attention(name, steps, warmup, device, backward=False):
         # dense-equivalent work: S recomputed, dP, dV, dK, dQ = 2.5 x the forward's two products
         from adasplash_amd import _attention
 
-        assert name in ("c4", "c3")
         # (as the autograd function does: the forward keeps the supports it found for the backward)
-        out, taus, bmask, supports = _attention.launch_forward(q, k, v, version=2, alpha=1.5, is_causal=True, niter=1,
-                                                               varlen=varlen, keep_supports=True)
+        if name == "c5":
+            kw, varlen = dict(alpha=1.333, is_causal=False), None
+            fwd_kw = dict(version=1, niter=10, **kw)
+        else:
+            kw = dict(alpha=1.5, is_causal=True)
+            fwd_kw = dict(version=2, niter=1, **kw)
+        out, taus, bmask, supports = _attention.launch_forward(q, k, v, varlen=varlen, keep_supports=True, **fwd_kw)
         dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(7)).to(q.dtype).to(device)
-        fn = lambda: _attention.launch_backward(q, k, v, dout, taus, bmask, alpha=1.5, is_causal=True,  # noqa: E731
-                                                varlen=varlen, supports=supports)
+        fn = lambda: _attention.launch_backward(q, k, v, dout, taus, bmask, varlen=varlen,  # noqa: E731
+                                                supports=supports, **kw)
         flops = 2.5 * flops
         cfg = dict(cfg, workload=cfg["workload"].replace("fwd", "bwd (dq, dk, dv)"))
-    if name == "c3" and not backward:
-        # a step of 0.35 ms: a short run would be timed while the clocks still ramp (the rows workloads do the same)
+    if (name == "c3" and not backward) or (name == "c5" and backward):
+        # a step of 0.35 ms (0.66 ms): a short run would be timed while the clocks still ramp (the rows workloads do the same)
         steps, warmup = max(steps, 100), max(warmup, 300)
     ms, wall_ms = _events_ms(fn, steps, warmup)
     tflops = flops / (ms * 1e-3) / 1e12
@@ -164,7 +172,7 @@ def bench_attention(name, steps, warmup, device, backward=False):
            "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS, "config": cfg}
     if name in ("c4", "c3") and not backward:
         res["tiles"] = v2_tile_stats(q, k, v, varlen)
-    if name == "c5":
+    if name == "c5" and not backward:
         from adasplash_amd.adasplash_block_mask import tile_sparsity
 
         _, total, active = tile_sparsity(q, k, v, alpha=1.333, is_causal=False, niter=10)
@@ -279,7 +287,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd", "c2_bwd"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd", "c5_bwd", "c2_bwd"])
     ap.add_argument("--no-extra", action="store_true", help="skip the entmax-rows and CPU-baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -332,9 +340,14 @@ def main():
                      "roofline": {"bound": "mfma", "achieved": res["eff_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                                   "unit": "TFLOP/s", "frac": res["frac_mfma_peak"],
                                   "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
-                                  "kernel": ("attn_bwd_dq_sparse_kernel + attn_bwd_dkdv_stream_kernel + dkdv_reduce_kernel" if args.workload == "c4_bwd" else "attn_bwd_dq_kernel + attn_bwd_dkdv_kernel") if bwd else FWD_KERNELS[args.workload],
+                                  "kernel": BWD_KERNELS[args.workload] if bwd else FWD_KERNELS[args.workload],
                                   "flops_per_launch": res["flops_per_step"]},
                      "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k == "wall_ms_per_step"}})
+        if bwd and args.workload != "c3_bwd":
+            # with the supports kept the sparse kernels issue no matrix products at all: the dense-equivalent rate
+            # says how fast a dense implementation would have to be, and may exceed the matrix pipe's peak
+            line["roofline"]["note"] = ("dense-equivalent FLOPs over time; the sparse-support kernels do this work on "
+                                        "the vector pipe and are bound by their gathers, so frac is not a utilisation")
         if "tiles" in res:
             line["tiles"] = res["tiles"]
         if not args.no_extra:
