@@ -41,12 +41,16 @@ static int head_dim_slot(int D) { return D == 16 ? 0 : (D == 32 ? 1 : (D == 64 ?
 
 // e4m3 copy of K for the first walk of the sparse-support forward: [B * Hkv][Npad][D] bytes in the order of K, values
 // beyond the format's range saturated, rows from N on zero.  A thread converts 16 values.  Heads the probe has marked
-// as dense are skipped (`hints`: two words per head).
+// as dense are skipped (`hints`: two words per head).  The values are multiplied by the head's power of two first
+// (`w1_scales`, from the probe).
+// (the first walk's operands lie on a grid of 1/16, see attn_sparse_kernel.h)
+#define G16(x) (((x) * ak + 786432.f) - 786432.f)
 template <typename T>
 __global__ __launch_bounds__(256) void k8_layout_kernel(const uint16_t* __restrict__ k, unsigned char* __restrict__ k8, int N,
-                                                       int Npad, int D, const uint32_t* hints) {
+                                                       int Npad, int D, const uint32_t* hints, const float* w1_scales) {
   const size_t head = blockIdx.y;
   if (hints[2 * head] >= (1u << 20)) return;
+  const float ak = w1_scales[2 * head + 1];
   const int per_row = D / 16;
   const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
   if (id >= (long long)Npad * per_row) return;
@@ -57,8 +61,8 @@ __global__ __launch_bounds__(256) void k8_layout_kernel(const uint16_t* __restri
     const u32x4 lo = *reinterpret_cast<const u32x4*>(src), hi = *reinterpret_cast<const u32x4*>(src + 8);
 #pragma unroll
     for (int e = 0; e < 4; e += 2) {
-      out[e >> 1] = cvt_e4m3_pair(unpack_lo<T>(lo[e + 1]), unpack_hi<T>(lo[e + 1]), cvt_e4m3_pair(unpack_lo<T>(lo[e]), unpack_hi<T>(lo[e]), 0u, false), true);
-      out[2 + (e >> 1)] = cvt_e4m3_pair(unpack_lo<T>(hi[e + 1]), unpack_hi<T>(hi[e + 1]), cvt_e4m3_pair(unpack_lo<T>(hi[e]), unpack_hi<T>(hi[e]), 0u, false), true);
+      out[e >> 1] = cvt_e4m3_pair(G16(unpack_lo<T>(lo[e + 1])), G16(unpack_hi<T>(lo[e + 1])), cvt_e4m3_pair(G16(unpack_lo<T>(lo[e])), G16(unpack_hi<T>(lo[e])), 0u, false), true);
+      out[2 + (e >> 1)] = cvt_e4m3_pair(G16(unpack_lo<T>(hi[e + 1])), G16(unpack_hi<T>(hi[e + 1])), cvt_e4m3_pair(G16(unpack_lo<T>(hi[e])), G16(unpack_hi<T>(hi[e])), 0u, false), true);
     }
   }
   *reinterpret_cast<u32x4*>(k8 + (head * (size_t)Npad + row) * D + c * 16) = out;
@@ -83,6 +87,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, int am) {
   __shared__ float qrows[4][256];
   __shared__ float red[4][2][4];
+  __shared__ float ksum[4];
   const int u = blockIdx.x, tid = threadIdx.x;
   const int units = p.B * p.Hkv;
   uint32_t* const ctrl = p.queue;
@@ -97,6 +102,7 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
     long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
     L = (int)(l < 0 ? 0 : (l > p.N ? p.N : l));
   }
+  if (p.w1_scales && tid < 2) p.w1_scales[2 * u + tid] = 1.f;
   if (L < 2048) return;  // short sequences: finding out in the kernel costs little
   int rows[4];
 #pragma unroll
@@ -111,11 +117,13 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
   const int key = (int)(((long long)tid * span) / 256);
   const uint16_t* krow = reinterpret_cast<const uint16_t*>(p.k) + ((size_t)(b * p.Hkv + kvh) * p.N + key) * D;
   float dot[4] = {0.f, 0.f, 0.f, 0.f};
+  float ksq = 0.f;
   for (int d = 0; d < D; d += 8) {
     const u32x4 w = *reinterpret_cast<const u32x4*>(krow + d);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float lo = unpack_lo<T>(w[e]), hi = unpack_hi<T>(w[e]);
+      ksq = fmaf(lo, lo, fmaf(hi, hi, ksq));
 #pragma unroll
       for (int j = 0; j < 4; ++j) dot[j] = fmaf(lo, qrows[j][d + 2 * e], fmaf(hi, qrows[j][d + 2 * e + 1], dot[j]));
     }
@@ -129,7 +137,27 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
       red[tid >> 6][1][j] = s2;
     }
   }
+  {
+    const float ks = wave_sum(ksq);
+    if ((tid & 63) == 0) ksum[tid >> 6] = ks;
+  }
   __syncthreads();
+  if (tid == 0 && p.w1_scales) {
+    // Scales of the first walk's operands: the sampled raw scores' root mean square goes to about 8 (the walk's
+    // tags hold scores up to 512), shared between q and k so that k's own root mean square comes near 8 / sqrt(D).
+    float raw2 = 0.f;
+    for (int j = 0; j < 4; ++j) raw2 += red[0][1][j] + red[1][1][j] + red[2][1][j] + red[3][1][j];
+    const float s_rms = sqrtf(raw2 / 1024.f) / p.qscale;
+    const float k_rms = sqrtf((ksum[0] + ksum[1] + ksum[2] + ksum[3]) / (256.f * (float)D));
+    if (s_rms > 0.f && k_rms > 0.f && s_rms < INFINITY && k_rms < INFINITY) {
+      const float a = exp2f(rintf(log2f(8.f / s_rms)));
+      float ak = exp2f(rintf(log2f(8.f / (sqrtf((float)D) * k_rms))));
+      ak = fminf(fmaxf(ak, 0x1p-40f), 0x1p40f);
+      float aq = fminf(fmaxf(a / ak, 0x1p-40f), 0x1p40f);
+      p.w1_scales[2 * u] = aq;
+      p.w1_scales[2 * u + 1] = ak;
+    }
+  }
   if (tid >= 4) return;
   {  // threads 0 .. 3: one sampled row each
     const int j = tid;
@@ -170,7 +198,7 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
 constexpr int kSparseMaxSlots = 1024;                       // workgroups of the persistent kernel
 constexpr size_t kSparseSlotBytes = (size_t)4 * 1616 * 8;   // four waves x 1616 candidates x (score, key)
 struct FwdWorkspace {
-  size_t vt_bytes, queue_off, flags_off, events_off, k8_off, total;
+  size_t vt_bytes, queue_off, scales_off, flags_off, events_off, k8_off, total;
   int slots;  // 0: no sparse-support kernel for these dimensions
 };
 static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
@@ -185,7 +213,9 @@ static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     if (slots > kSparseMaxSlots) slots = kSparseMaxSlots;
     w.slots = (int)slots;
     w.queue_off = align256(w.vt_bytes);
-    w.flags_off = align256(w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8);  // eight counters, then two hint words per K/V head and two more
+    // eight counters, then two hint words per K/V head and two more, then two scales per K/V head
+    w.scales_off = w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8;
+    w.flags_off = align256(w.scales_off + (size_t)B * Hkv * 8);
     w.events_off = align256(w.flags_off + (size_t)items * 4);
     w.k8_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
     w.total = w.k8_off + (size_t)B * Hkv * npad_of(N) * D;  // the e4m3 copy of K
@@ -275,6 +305,7 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.hints = nullptr;
   p.events = nullptr;
   p.k8 = nullptr;
+  p.w1_scales = nullptr;
   p.save_flags = nullptr;
   p.save_lens = nullptr;
   p.save_tshift = nullptr;
@@ -298,6 +329,7 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
       p.block_flags = (int32_t*)(ws + w.flags_off);
       p.events = ws + w.events_off;
       p.k8 = ws + w.k8_off;
+      p.w1_scales = (float*)(ws + w.scales_off);
       if (sl.total) {
         unsigned char* sp = (unsigned char*)supports;
         p.save_flags = (int32_t*)(sp + sl.flags_off);
@@ -308,10 +340,10 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
       const dim3 k8_grid((unsigned)(((long long)p.Npad * (D / 16) + 255) / 256), (unsigned)(B * Hkv));
       if (dtype == ADSP_BF16) {
         hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
-        hipLaunchKernelGGL(k8_layout_kernel<bf16_t>, k8_grid, dim3(256), 0, s, (const uint16_t*)k, ws + w.k8_off, N, p.Npad, D, (const uint32_t*)p.hints);
+        hipLaunchKernelGGL(k8_layout_kernel<bf16_t>, k8_grid, dim3(256), 0, s, (const uint16_t*)k, ws + w.k8_off, N, p.Npad, D, (const uint32_t*)p.hints, (const float*)p.w1_scales);
       } else {
         hipLaunchKernelGGL(attn_probe_kernel<f16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, p, D, am);
-        hipLaunchKernelGGL(k8_layout_kernel<f16_t>, k8_grid, dim3(256), 0, s, (const uint16_t*)k, ws + w.k8_off, N, p.Npad, D, (const uint32_t*)p.hints);
+        hipLaunchKernelGGL(k8_layout_kernel<f16_t>, k8_grid, dim3(256), 0, s, (const uint16_t*)k, ws + w.k8_off, N, p.Npad, D, (const uint32_t*)p.hints, (const float*)p.w1_scales);
       }
       int rc = dtype == ADSP_BF16 ? (D == 64 ? launch_attn_sparse_bf16_d64(p, am, w.slots, s) : launch_attn_sparse_bf16_d128(p, am, w.slots, s))
                                   : (D == 64 ? launch_attn_sparse_f16_d64(p, am, w.slots, s) : launch_attn_sparse_f16_d128(p, am, w.slots, s));

@@ -41,6 +41,9 @@ struct AttnParams {
   uint32_t* hints;        // [B * Hkv + 1][2] row blocks {given up, served} per K/V head, then over all heads; zero at launch
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
   const unsigned char* k8;  // fp8 (e4m3) copy of K, [B * Hkv][Npad][D] bytes, rows past N zero: the operand of the first walk
+  // Powers of two per K/V head, {for q, for k}, set by the probe: q and k are multiplied by them before they are
+  // rounded for the first walk, so that its scores stay inside the range its position tags need (null: 1, 1)
+  float* w1_scales;
   // Supports kept for the backward (null: none kept).  The sparse-support kernel then writes its candidate streams to a
   // place of their own per (row block, wave) and leaves them there, with their lengths, every row's threshold minus
   // lower bound (raw score units: an entry is a member of the support when its value exceeds it), and a flag per row

@@ -7,12 +7,15 @@
 //
 //   walk 1  S^T = K Q^T per tile on the fp8 MFMA (twice the 16-bit rate, half the tile bytes) from an e4m3 copy of K
 //           and Q fragments rounded the same way; a lane keeps the four largest block maxima of its half of the row's
-//           keys together with the keys they belong to (the key's position rides in the low mantissa bits).  These
-//           scores are approximate and only choose keys: the scores of the eight chosen keys of a row are then
-//           recomputed from the 16-bit inputs.  The threshold of any subset of a row's scores is a lower bound of the
-//           row's threshold (f only grows when entries are added), so a few Newton steps from the left on those eight
-//           values give a lower bound `lo` that lies within a few hundredths (in z) of the threshold for such rows,
-//           whichever keys were chosen.
+//           keys together with the keys they belong to.  Both operands are first put on a grid of 1/16, so every
+//           product is a multiple of 2^-8 and the sums are exact in fp32; the accumulators start at 1536 + i 2^-13 for
+//           the lane's i-th value of a block, which leaves i in the four lowest mantissa bits of every score: the
+//           maximum of a block knows its key without an instruction per score.  These scores are approximate and only
+//           choose keys (a wrong position, should the exactness ever fail, is a poor choice and no more): the scores
+//           of the eight chosen keys of a row are then recomputed from the 16-bit inputs.  The threshold of any subset
+//           of a row's scores is a lower bound of the row's threshold (f only grows when entries are added), so a few
+//           Newton steps from the left on those eight values give a lower bound `lo` that lies within a few
+//           hundredths (in z) of the threshold for such rows, whichever keys were chosen.
 //   walk 2  the same products with the accumulators preloaded with -lo; a lane whose eight scores of a 16-key half
 //           block have a positive maximum writes those eight values and the half block's index to its event list in
 //           global memory (a per-workgroup slot of the workspace; the events are a few per cent of the scores).
@@ -38,6 +41,12 @@ namespace adsp {
 #endif
 #ifndef ADSP_SPARSE_WAVES
 #define ADSP_SPARSE_WAVES 4
+#endif
+// Profiling builds only (-DADSP_SPARSE_STOP=n in the build's extra flags): a row block ends behind its first walk (1),
+// the lower bound (2), the second walk (3) or the thresholds (4), so that the stages can be timed by difference.  Such
+// a build computes no output.
+#ifndef ADSP_SPARSE_STOP
+#define ADSP_SPARSE_STOP 0
 #endif
 constexpr int kSparseStreamCap = 1616;  // candidates per wave the workspace slot holds (SparseGeo::kListCap is at most this)
 constexpr int kSparseMaxKeys = 65536;   // the lists hold 16-bit key indices
@@ -68,6 +77,20 @@ __device__ __forceinline__ f32x16 mfma_fp8(u32x4 a_lo, u32x4 a_hi, const uint32_
   const i32x8 a = {(int)a_lo[0], (int)a_lo[1], (int)a_lo[2], (int)a_lo[3], (int)a_hi[0], (int)a_hi[1], (int)a_hi[2], (int)a_hi[3]};
   const i32x8 bb = {(int)b[0], (int)b[1], (int)b[2], (int)b[3], (int)b[4], (int)b[5], (int)b[6], (int)b[7]};
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, bb, c, 0, 0, 0, 0, 0, 0);  // both operands e4m3, no block scales
+}
+
+// median of three unsigned values
+__device__ __forceinline__ uint32_t umed3(uint32_t a, uint32_t b, uint32_t c) {
+  uint32_t r;
+  asm("v_med3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// First walk: a score past a row's last valid key (0 lies below every real one, which start at 1024), and the
+// rounding of an operand to a multiple of 1/16 (the sum with 1.5 * 2^19 has its last place there).
+constexpr float kW1Masked = 0.f;
+__device__ __forceinline__ float grid16(float x) {
+  const float c = 786432.f;
+  return (x + c) - c;
 }
 
 // inclusive prefix sum over the wave on the DPP network; all 64 lanes active
@@ -253,6 +276,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // values [32 lh, 32 lh + 32) of its row, in the order of the copy of K.  Rows past the valid length are zero
     // (their scores are never used). ------------------------------------------------------------------------------
     const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
+    const float aq = p.w1_scales[2 * (b * p.Hkv + kvh)], aqk = aq * p.w1_scales[2 * (b * p.Hkv + kvh) + 1];
     uint32_t q8[D / 64 * 8];
     uint32_t qf[G::kQRegs];  // those of the 16-bit products: loaded behind the first walk
 #pragma unroll
@@ -262,8 +286,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + c * 64 + lh * 32 + hq * 8);
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
-          uint32_t w = cvt_e4m3_pair(unpack_lo<T>(raw[e]), unpack_hi<T>(raw[e]), 0u, false);
-          w = cvt_e4m3_pair(unpack_lo<T>(raw[e + 1]), unpack_hi<T>(raw[e + 1]), w, true);
+          uint32_t w = cvt_e4m3_pair(grid16(aq * unpack_lo<T>(raw[e])), grid16(aq * unpack_hi<T>(raw[e])), 0u, false);
+          w = cvt_e4m3_pair(grid16(aq * unpack_lo<T>(raw[e + 1])), grid16(aq * unpack_hi<T>(raw[e + 1])), w, true);
           q8[c * 8 + hq * 2 + (e >> 1)] = live ? w : 0u;
         }
       }
@@ -323,16 +347,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         stage = stage + 1 == kStages ? 0 : stage + 1;
       }
     };
-    // approximate S^T of one tile from the fp8 operands; f(s0, s1) unless no row of the wave sees the tile.  Scores past
-    // a row's last valid key are hugely negative (finite: a position is still to be written into their low bits).
+    // accumulator start values of the first walk (opaque to the compiler: they must stay in registers)
+    float ctag[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      ctag[i] = 1536.f + (float)i * (1.f / 8192.f);
+      asm volatile("" : "+v"(ctag[i]));
+    }
+    // approximate S^T of one tile from the fp8 operands; f(s0, s1) unless no row of the wave sees the tile.  A score
+    // is 1536 + (the sum of the products, a multiple of 2^-8 below 512 in size) + (its index among the lane's 16
+    // values of the block) 2^-13: a float in [1024, 2048) whose mantissa holds the index in bits 0 .. 3 and the sum
+    // from bit 5 on.  Scores past a row's last valid key are 0.
     auto for_tile8 = [&](int kt, const unsigned char* kt_lds, auto&& f) {
       if (p.causal && kt * kBN > wave_row0 + 31) return;
       const bool need_mask = (kt * kBN + kBN - 1 > L - 1) || (p.causal && kt * kBN + kBN - 1 > wave_row0);
       f32x16 s0, s1;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        s0[i] = 0.f;
-        s1[i] = 0.f;
+        s0[i] = ctag[i];
+        s1[i] = ctag[i];
       }
       uint32_t ka = (uint32_t)(uintptr_t)kt_lds + k8_lane;
       asm volatile("" : "+v"(ka));
@@ -349,8 +382,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         const int jb = kt * kBN + 4 * lh;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          s0[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? s0[i] : -1e30f;
-          s1[i] = (jb + 32 + 8 * (i >> 2) + (i & 3) <= lim) ? s1[i] : -1e30f;
+          s0[i] = (jb + 8 * (i >> 2) + (i & 3) <= lim) ? s0[i] : kW1Masked;
+          s1[i] = (jb + 32 + 8 * (i >> 2) + (i & 3) <= lim) ? s1[i] : kW1Masked;
         }
       }
       f(s0, s1);
@@ -403,38 +436,39 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     };
 
     // ---- walk 1: the four largest block maxima of the lane's keys ---------------------------------------------
-    float t1 = -INFINITY, t2 = -INFINITY, t3 = -INFINITY, t4 = -INFINITY;
-    auto keep_top = [&](float x) {
-      const float n2 = __builtin_amdgcn_fmed3f(t1, t2, x), n3 = __builtin_amdgcn_fmed3f(t2, t3, x), n4 = __builtin_amdgcn_fmed3f(t3, t4, x);
-      t1 = fmaxf(t1, x);
-      t2 = n2;
-      t3 = n3;
-      t4 = n4;
-    };
+    // A block maximum becomes a 29-bit word: the sum in steps of 1/16 (14 bits), the 32-key block (11 bits), the
+    // position in the block (4 bits); unsigned comparisons order the words by their sums.  Words whose sum field is
+    // 0 (nothing seen, or only masked scores) stand for no key.
     // A flat score distribution (a support of hundreds of keys) shows early: most block maxima lie close to the
     // running maximum.  Tiles 6 .. 11 are counted; if more than half of their (lane, block) maxima lie within 1/4 (in
     // z) of the lane's running maximum, the row block is given up before the walk is over.  A heuristic that only
     // decides which kernel does the work.
+    uint32_t t1 = 0u, t2 = 0u, t3 = 0u, t4 = 0u;
+    auto keep_top = [&](uint32_t x) {
+      const uint32_t n2 = umed3(t1, t2, x), n3 = umed3(t2, t3, x), n4 = umed3(t3, t4, x);
+      t1 = t1 > x ? t1 : x;
+      t2 = n2;
+      t3 = n3;
+      t4 = n4;
+    };
     int near_cnt = 0;
-    // A score carries its position in the low 15 bits of its mantissa (4: which of the lane's 16 values of the block,
-    // 11: the 32-key block), so the maxima know their keys at the price of one instruction per score; the approximate
-    // scores have fewer than nine good mantissa bits anyway.
-    auto tagged = [](float x, uint32_t bits, uint32_t tag) { return __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, x) & ~bits) | tag); };
+    const uint32_t near_d = (uint32_t)fminf(0.25f * inv_qs * 16.f * aqk, 8191.f) << 15;
     walk(std::integral_constant<int, SG::kStages8>{}, std::integral_constant<int, SG::kK8Tile>{}, std::integral_constant<int, kK8Per>{}, issue_k8, [&](int kt, const unsigned char* kt_lds) {
       for_tile8(kt, kt_lds, [&](const f32x16& s0, const f32x16& s1) {
-        float m0v = tagged(s0[0], 15u, 0u), m1v = tagged(s1[0], 15u, 0u);
+        float m0v = fmaxf(s0[0], s0[1]), m1v = fmaxf(s1[0], s1[1]);
 #pragma unroll
-        for (int i = 1; i < 16; ++i) {
-          m0v = fmaxf(m0v, tagged(s0[i], 15u, (uint32_t)i));
-          m1v = fmaxf(m1v, tagged(s1[i], 15u, (uint32_t)i));
+        for (int i = 2; i < 16; i += 2) {
+          m0v = fmaxf(fmaxf(m0v, s0[i]), s0[i + 1]);
+          m1v = fmaxf(fmaxf(m1v, s1[i]), s1[i + 1]);
         }
-        m0v = tagged(m0v, 0x7ff0u, (uint32_t)(2 * kt) << 4);
-        m1v = tagged(m1v, 0x7ff0u, (uint32_t)(2 * kt + 1) << 4);
-        keep_top(m0v);
-        keep_top(m1v);
+        const uint32_t b0 = __builtin_bit_cast(uint32_t, m0v), b1 = __builtin_bit_cast(uint32_t, m1v);
+        const uint32_t k0 = (((b0 >> 9) & 0x3fffu) << 15) | ((b0 & 15u) | ((uint32_t)(2 * kt) << 4));
+        const uint32_t k1 = (((b1 >> 9) & 0x3fffu) << 15) | ((b1 & 15u) | ((uint32_t)(2 * kt + 1) << 4));
+        keep_top(k0);
+        keep_top(k1);
         if (kt >= 6 && kt < 12) {
-          const float near = t1 - 0.25f * inv_qs;
-          near_cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && m0v > near)) + __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && m1v > near));
+          const uint32_t near = t1 > near_d ? t1 - near_d : 0u;
+          near_cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && k0 > near)) + __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && k1 > near));
           if (kt == 11 && near_cnt > 6 * 128 / 2 && lane == 0) s_giveup[1] = 1u;
         }
       });
@@ -450,6 +484,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
       continue;
     }
+#if ADSP_SPARSE_STOP == 1
+    continue;
+#endif
     // ---- lower bound of the row's threshold from its eight kept values (raw score units) --------------------
     // f(t) = qs^2 sum (r - t)_+^2 - 1 (alpha 1.5) or qs sum (r - t)_+ - 1 (alpha 2) is convex and decreasing and
     // f(max - 1 / qs) >= 0, so Newton from there approaches the subset's root from the left and never passes it.
@@ -466,45 +503,69 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // ----------------------------------------------------------------------------------------------------------------
     float r[8];
     {
-      const uint32_t u[4] = {__builtin_bit_cast(uint32_t, t1), __builtin_bit_cast(uint32_t, t2), __builtin_bit_cast(uint32_t, t3), __builtin_bit_cast(uint32_t, t4)};
-      uint32_t pu[4];
+      // The rows of the chosen keys are gathered into LDS the way the walks' tiles get there: per product m the wave
+      // loads a 32-row "tile" whose row i is the key that row i chose as its m-th, with 1 KB DMA instructions (a
+      // group of kC lanes per key row: whole rows, coalesced), and reads the A fragments from it as from a K tile.
+      const uint32_t u[4] = {t1, t2, t3, t4};
+      constexpr int kRowsPer = 64 / KS::kC;   // key rows per 1 KB DMA instruction
+      constexpr int kInstr = 32 / kRowsPer;   // instructions per gathered tile
+      uint32_t* const ktab = reinterpret_cast<uint32_t*>(lds_all + SG::kStages * G::kKTile + wave * SG::kRingBytes);  // [8][kRowsPer][kInstr]
+      unsigned char* const gtile = lds_all + wave * (32 * G::kKRow);
+      bool okm[4], okp[4];
 #pragma unroll
-      for (int m = 0; m < 4; ++m) pu[m] = (uint32_t)__shfl_xor((int)u[m], 32, 64);
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t w = u[i];
+        okm[i] = (w >> 15) != 0u;
+        uint32_t key = ((w >> 4) & 0x7ffu) * 32u + 8u * ((w & 15u) >> 2) + (w & 3u) + 4u * (uint32_t)lh;
+        // (a position that did not survive -- sums beyond the tags' range -- may name a key the row does not see: only
+        // scores of the row's own keys bound its threshold)
+        okm[i] = okm[i] && (int)key <= lim;
+        key = okm[i] ? key : 0u;
+        ktab[(4 * lh + i) * 32 + (lq % kRowsPer) * kInstr + lq / kRowsPer] = key;
+        okp[i] = __shfl_xor((int)okm[i], 32, 64) != 0;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
       const int diag = ((lq >> 3) << 2) | (lq & 3);  // which of the lane's 16 values of a block belongs to key lq of the block,
       const bool diag_here = lh == ((lq >> 2) & 1);  // and which of the row's two lanes holds it
-      constexpr int kBatch = D / 16;
+      const unsigned char* kg = uniform_ptr(kglob);
+      const int grow = lane / KS::kC, gslot = lane % KS::kC;
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        // the row's first lane chose keys 0 .. 3, its second lane keys 4 .. 7
-        const uint32_t w = ((m < 4) == (lh == 0)) ? u[m & 3] : pu[m & 3];
-        const bool ok = __builtin_bit_cast(float, w) > -1e29f;  // fewer than four valid keys leave -inf or masked entries behind
-        uint32_t key = ((w >> 4) & 0x7ffu) * 32u + 8u * ((w & 15u) >> 2) + (w & 3u) + (m < 4 ? 0u : 4u);
-        key = (ok && key < (uint32_t)N) ? key : 0u;
-        const unsigned char* krow = kglob + (size_t)key * G::kKRow + 16 * lh;
+        uint32_t keys[kInstr];
+#pragma unroll
+        for (int j = 0; j < kInstr; j += 4) {
+          const u32x4 kk = *reinterpret_cast<const u32x4*>(&ktab[m * 32 + grow * kInstr + j]);
+          keys[j] = kk[0];
+          keys[j + 1] = kk[1];
+          keys[j + 2] = kk[2];
+          keys[j + 3] = kk[3];
+        }
+#pragma unroll
+        for (int j = 0; j < kInstr; ++j) {
+          const int rr = j * kRowsPer + grow;
+          dma16s(kg, keys[j] * (uint32_t)G::kKRow + (uint32_t)((gslot ^ KS::sw(rr)) << 4), gtile + j * 1024);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the gathered tile is in LDS (this wave's own loads)
         f32x16 acc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        uint32_t ka = (uint32_t)(uintptr_t)gtile + k_lane;
+        asm volatile("" : "+v"(ka));
+        u32x4 af[D / 16];
 #pragma unroll
-        for (int k0 = 0; k0 < D / 16; k0 += kBatch) {
-          u32x4 kv[kBatch];
+        for (int ks = 0; ks < D / 16; ++ks) af[ks] = lds_read16(ka ^ (ks << 5));
 #pragma unroll
-          for (int j = 0; j < kBatch; ++j) kv[j] = *reinterpret_cast<const u32x4*>(krow + (k0 + j) * 32);
-#pragma unroll
-          for (int j = 0; j < kBatch; ++j) {
-            const int ks = k0 + j;
-            acc = mfma_16bit<T>(kv[j], u32x4{qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]}, acc);
-          }
-        }
-        // (the order of issue: a key's loads together, then its products)
-        __builtin_amdgcn_sched_group_barrier(0x020, D / 16, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, D / 16, 0);
+        for (int ks = 0; ks < D / 16; ++ks) acc = mfma_16bit<T>(af[ks], u32x4{qf[ks * 4], qf[ks * 4 + 1], qf[ks * 4 + 2], qf[ks * 4 + 3]}, acc);
         float d = acc[0];
 #pragma unroll
         for (int i = 1; i < 16; ++i) d = diag == i ? acc[i] : d;
         const float other = __shfl_xor(d, 32, 64);
         d = diag_here ? d : other;
+        const bool ok = ((m < 4) == (lh == 0)) ? okm[m & 3] : okp[m & 3];
         r[m] = ok ? d : -INFINITY;
       }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the last fragment reads are done before the tiles of walk 2 arrive
     }
     float lo_raw;
     {
@@ -537,9 +598,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
       // the margin covers the rounding of the iteration; rows past the valid length take no part in walk 2
       lo_raw = t - (1e-5f * inv_qs + 1e-6f * fabsf(rmax));
+      // (a row none of whose chosen keys could be used -- its first walk's sums left the tags' range -- has no bound:
+      // the row block goes to the dense kernel; the second walk stops at its first tile)
+      if (live && !(rmax > -INFINITY)) s_giveup[1] = 1u;
       lo_raw = (live && rmax > -INFINITY) ? lo_raw : INFINITY;
     }
 
+#if ADSP_SPARSE_STOP == 2
+    if (lo_raw == 12345.f) p.taus[qi] = lo_raw;  // (keeps the bound alive)
+    continue;
+#endif
     // ---- walk 2: collect the scores above the bound -------------------------------------------------------------
     // A lane whose eight scores of a 16-key half block have a positive maximum puts them, with a tag, into the wave's
     // ring in LDS (slots are handed out with a ballot: no atomics).  When the ring is full the wave empties it, one
@@ -614,6 +682,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
     };
+    // One decision per tile: the four half blocks' events are counted together; when they fit the ring (after a flush
+    // if need be) every lane writes its events at slots known from the four ballots, without further tests.  A tile
+    // with more events than the ring holds (the first tiles of a sequence) goes through in eight parts.
+    auto put_at = [&](unsigned long long m, bool mine, const f32x16& s, int first, uint32_t tag, int base) {
+      if (mine) {
+        const int slot = base + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        f32x4 w0 = {s[first], s[first + 1], s[first + 2], s[first + 3]};
+        f32x4 w1 = {s[first + 4], s[first + 5], s[first + 6], s[first + 7]};
+        *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
+        *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
+        ring_tag[slot] = (tag << 6) | (uint32_t)lane;
+      }
+    };
     walk(std::integral_constant<int, SG::kStages>{}, std::integral_constant<int, G::kKTile>{}, std::integral_constant<int, kKPer>{}, issue_k, [&](int kt, const unsigned char* kt_lds) {
       for_tile(kt, kt_lds, -lo_raw, [&](const f32x16& s0, const f32x16& s1) {
         float h00 = s0[0], h01 = s0[8], h10 = s1[0], h11 = s1[8];
@@ -624,10 +705,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           h10 = fmaxf(h10, s1[i]);
           h11 = fmaxf(h11, s1[8 + i]);
         }
-        collect(s0, 0, h00, (uint32_t)(kt * 4 + 0), kt);
-        collect(s0, 8, h01, (uint32_t)(kt * 4 + 1), kt);
-        collect(s1, 0, h10, (uint32_t)(kt * 4 + 2), kt);
-        collect(s1, 8, h11, (uint32_t)(kt * 4 + 3), kt);
+        const unsigned long long m0 = __builtin_amdgcn_ballot_w64(h00 > 0.f), m1 = __builtin_amdgcn_ballot_w64(h01 > 0.f);
+        const unsigned long long m2 = __builtin_amdgcn_ballot_w64(h10 > 0.f), m3 = __builtin_amdgcn_ballot_w64(h11 > 0.f);
+        const int c0 = __builtin_popcountll(m0), c1 = __builtin_popcountll(m1), c2 = __builtin_popcountll(m2), c3 = __builtin_popcountll(m3);
+        const int E = c0 + c1 + c2 + c3;
+        if (E != 0) {
+          int step = E <= SG::kRing ? -1 : 0;
+          do {
+            unsigned long long sub = 0ull;
+            int need = E;
+            if (step >= 0) {
+              const int hb = step >> 1;
+              sub = hb == 0 ? m0 : hb == 1 ? m1 : hb == 2 ? m2 : m3;
+              sub &= (step & 1) ? ~0xffffffffull : 0xffffffffull;
+              need = __builtin_popcountll(sub);
+            }
+            if (ring_n + need > SG::kRing) flush(kt & 1, kt);
+            if (step < 0) {
+              put_at(m0, h00 > 0.f, s0, 0, (uint32_t)(kt * 4 + 0), ring_n);
+              put_at(m1, h01 > 0.f, s0, 8, (uint32_t)(kt * 4 + 1), ring_n + c0);
+              put_at(m2, h10 > 0.f, s1, 0, (uint32_t)(kt * 4 + 2), ring_n + c0 + c1);
+              put_at(m3, h11 > 0.f, s1, 8, (uint32_t)(kt * 4 + 3), ring_n + c0 + c1 + c2);
+              step = 8;
+            } else {
+              const int hb = step >> 1;
+              if ((sub >> lane) & 1ull) {
+                f32x4 w0, w1;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                  w0[i] = hb == 0 ? s0[i] : hb == 1 ? s0[8 + i] : hb == 2 ? s1[i] : s1[8 + i];
+                  w1[i] = hb == 0 ? s0[4 + i] : hb == 1 ? s0[12 + i] : hb == 2 ? s1[4 + i] : s1[12 + i];
+                }
+                const int slot = ring_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(sub >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)sub, 0u));
+                *reinterpret_cast<f32x4*>(ring + slot * 8) = w0;
+                *reinterpret_cast<f32x4*>(ring + slot * 8 + 4) = w1;
+                ring_tag[slot] = ((uint32_t)(kt * 4 + hb) << 6) | (uint32_t)lane;
+              }
+              ++step;
+            }
+            ring_n += need;
+          } while (step < 8);
+        }
       });
     });
     flush(0, nt);
@@ -643,6 +761,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       continue;
     }
 
+#if ADSP_SPARSE_STOP == 3
+    continue;
+#endif
     // ---- the wave's stream -> per-row lists in its share of LDS (a counting sort by row) ----------------------------
     unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
     float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap scores, later probabilities
@@ -744,6 +865,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
     }
 
+#if ADSP_SPARSE_STOP == 4
+    continue;
+#endif
     // ---- output: a group of D / 8 lanes per row, each lane 8 columns; the V rows of a row's support are fetched
     // kDepth at a time (all in flight together), weighted, summed, and the row is stored with 16-byte accesses.  The
     // weights enter the two-term dot product as (p, 0) and (0, p) pairs of the element type, i.e. rounded to it, as
