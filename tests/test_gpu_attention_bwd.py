@@ -270,9 +270,9 @@ def test_full_size_gqa_varlen_backward():
     """The headline workload's backward at full size (B=8, Hq=32, Hkv=8, N=8192, D=128, bf16, ragged lengths): the
     gradients of padded rows and keys are zero; one whole K/V head of the shortest sequence (its four query heads)
     meets the oracle; and the two independent routes - fp32 arithmetic on the kept supports, the dense MFMA kernels -
-    agree everywhere within twice the bound each is held to against the oracle.  niter = 10: with a single solver step
-    the dense forward's threshold is off by up to 6e-3 on rows whose support is one large and a dozen tiny
-    probabilities, which doubles those tiny weights in its backward (the sparse route solves to convergence)."""
+    agree everywhere within twice the bound each is held to against the oracle.  niter = 1, the API's default: the
+    sparse route solves to convergence whatever niter is, and the dense kernel serving a call alone takes the
+    reference's extra update behind its niter steps (adasplash/adasplash_v2.py:617-681)."""
     g = torch.Generator().manual_seed(11)
     B, Hq, Hkv, N, D = 8, 32, 8, 8192, 128
     dt = torch.bfloat16
@@ -282,7 +282,7 @@ def test_full_size_gqa_varlen_backward():
     do = torch.randn(B, Hq, N, D, generator=g).to(dt).to(DEV)
     lens = [7297, 6553, 5730, 1500, 6310, 4494, 8192, 4555]
     vl = torch.tensor(lens, dtype=torch.int32, device=DEV)
-    sparse, dense = _both_routes(q, k, v, do, lambda a, b, c: A.adasplash_v2(a, b, c, niter=10, varlen=vl))
+    sparse, dense = _both_routes(q, k, v, do, lambda a, b, c: A.adasplash_v2(a, b, c, niter=1, varlen=vl))
     for got in (sparse, dense):
         for t in got:
             assert torch.isfinite(t.float()).all()
