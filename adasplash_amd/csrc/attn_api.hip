@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void k8_layout_kernel(const uint16_t* __restri
                                                        int Npad, int D, const uint32_t* hints, const float* w1_scales) {
   const size_t head = blockIdx.y;
   if (hints[2 * head] >= (1u << 20)) return;
-  const float ak = w1_scales[2 * head + 1];
+  const float ak = w1_scales[4 * head + 1];
   const int per_row = D / 16;
   const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
   if (id >= (long long)Npad * per_row) return;
@@ -73,16 +73,19 @@ static int mblocks_of(int N) { return (N + kMaskRows - 1) / kMaskRows; }
 static int mask_words_of(int N) { return ((N + kBN - 1) / kBN + 31) / 32; }
 
 // Control words of the sparse-support forward (the `queue` pointer of AttnParams): eight work counters, the number
-// of row blocks it left to the dense kernel, a word saying that the probe below predicts every K/V head to be dense; from word
-// 64 on two hint counters {given up, served} per K/V head and one more pair over all heads.
+// of row blocks it left to the dense kernel, a word saying that the probe below leaves every K/V head to the dense
+// kernel; from word 64 on two words per K/V head and two more (the first of a head's pair is 1 << 20 when the probe
+// leaves the whole head to the dense kernel; the backward's kernels keep row-block counters in the others), then four
+// floats per K/V head (AttnParams::w1_scales).
 //
 // attn_probe_kernel clears them and looks at a sample of each K/V head's scores (one workgroup per head: four long
-// query rows of the group's first head against 256 evenly spaced keys): from the sample's variance and the row
-// length, the support a Gaussian score distribution would have follows in closed form (n s^2 g(a) = 1 with
+// query rows of the group's first head against 256 evenly spaced keys): from the sample's variance the support a
+// Gaussian score distribution would have for a row that sees n keys follows in closed form (n s^2 g(a) = 1 with
 // g(a) = (1 + a^2) Q(a) - a phi(a) for alpha = 1.5, n s h(a) = 1 with h(a) = phi(a) - a Q(a) for alpha = 2; support
-// n Q(a)).  Heads whose predicted support is far beyond what the candidate lists hold are marked as given up, so the
-// sparse-support kernel does not spend a walk on finding that out.  The prediction only decides which kernel does
-// the work; a head it gets wrong is caught by the kernel's own checks.
+// n Q(a)).  It grows with n: the probe stores the largest n whose predicted support the candidate lists hold, and the
+// sparse-support kernels leave the row blocks that see more keys to the dense kernels without spending a walk on
+// them.  The prediction only decides which kernel does the work (a row block it gets wrong is caught by the kernel's
+// own checks), and it depends on the inputs alone: the same call takes the same way every time.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, int am) {
   __shared__ float qrows[4][256];
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
   const int u = blockIdx.x, tid = threadIdx.x;
   const int units = p.B * p.Hkv;
   uint32_t* const ctrl = p.queue;
-  if (u == 0 && tid < 10) ctrl[tid] = 0u;
+  if (u == 0 && tid < 11) ctrl[tid] = 0u;
   if (u == 0 && tid < 2) ctrl[64 + 2 * units + tid] = 0u;
   if (tid < 2) ctrl[64 + 2 * u + tid] = 0u;
   const int b = u / p.Hkv, kvh = u % p.Hkv, group = p.Hq / p.Hkv;
@@ -102,8 +105,8 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
     long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
     L = (int)(l < 0 ? 0 : (l > p.N ? p.N : l));
   }
-  if (p.w1_scales && tid < 2) p.w1_scales[2 * u + tid] = 1.f;
-  if (L < 2048) return;  // short sequences: finding out in the kernel costs little
+  if (p.w1_scales && tid < 4) p.w1_scales[4 * u + tid] = tid < 2 ? 1.f : (tid == 2 ? INFINITY : 0.f);
+  if (L < 256) return;  // short sequences: finding out in the kernel costs little
   int rows[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) rows[j] = L - 1 - j * (L / 16);
@@ -154,42 +157,56 @@ __global__ __launch_bounds__(256) void attn_probe_kernel(AttnParams p, int D, in
       float ak = exp2f(rintf(log2f(8.f / (sqrtf((float)D) * k_rms))));
       ak = fminf(fmaxf(ak, 0x1p-40f), 0x1p40f);
       float aq = fminf(fmaxf(a / ak, 0x1p-40f), 0x1p40f);
-      p.w1_scales[2 * u] = aq;
-      p.w1_scales[2 * u + 1] = ak;
+      p.w1_scales[4 * u] = aq;
+      p.w1_scales[4 * u + 1] = ak;
     }
   }
-  if (tid >= 4) return;
-  {  // threads 0 .. 3: one sampled row each
-    const int j = tid;
+  if (tid >= 64) return;
+  // The first wave: the score spread pooled over the four sampled rows, and for 64 row lengths n (a geometric grid from
+  // 64 to a million keys, one per lane) the support a Gaussian score distribution of that spread would have.  The
+  // prediction grows with n; the largest n whose support still fits is what the sparse-support kernels compare a row
+  // block's keys with.
+  float var = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
     const float s1 = red[0][0][j] + red[1][0][j] + red[2][0][j] + red[3][0][j];
     const float s2 = red[0][1][j] + red[1][1][j] + red[2][1][j] + red[3][1][j];
-    const float mean = s1 / 256.f, var = fmaxf(s2 / 256.f - mean * mean, 0.f), sd = sqrtf(var);
-    const float n = (float)(p.causal ? rows[j] + 1 : L);
-    float lo = -2.f, hi = 7.f;
-    for (int it = 0; it < 14; ++it) {
-      const float a = 0.5f * (lo + hi);
-      const float Q = 0.5f * erfcf(a * 0.70710678f), phi = 0.39894228f * __expf(-0.5f * a * a);
-      float f;
-      if (am == ATT_2) f = n * sd * (phi - a * Q);
-      else if (am == ATT_15) f = n * var * ((1.f + a * a) * Q - a * phi);
-      else {  // any alpha: n E[(sd (Z - a))_+^c0] by the midpoint rule over [a, a + 8]
-        float acc = 0.f;
-        for (int i = 0; i < 32; ++i) {
-          const float x = 0.25f * ((float)i + 0.5f);
-          acc += __expf(p.c0 * __logf(sd * x)) * 0.39894228f * __expf(-0.5f * (a + x) * (a + x));
-        }
-        f = n * acc * 0.25f;
-      }
-      if (f > 1.f) lo = a;
-      else hi = a;
-    }
-    const float support = n * 0.5f * erfcf(0.5f * (lo + hi) * 0.70710678f);
-    red[0][0][j] = support > 40.f ? 1.f : 0.f;
+    const float mean = s1 / 256.f;
+    var += 0.25f * fmaxf(s2 / 256.f - mean * mean, 0.f);
   }
-  // (the four threads are lanes of one wave: their LDS writes are in order before the read below)
-  const int dense_rows = (int)(red[0][0][0] + red[0][0][1] + red[0][0][2] + red[0][0][3]);
+  const float sd = sqrtf(var);
+  const float n = 64.f * exp2f((float)tid * (14.f / 63.f));
+  float lo = -2.f, hi = 7.f;
+  for (int it = 0; it < 14; ++it) {
+    const float a = 0.5f * (lo + hi);
+    const float Q = 0.5f * erfcf(a * 0.70710678f), phi = 0.39894228f * __expf(-0.5f * a * a);
+    float f;
+    if (am == ATT_2) f = n * sd * (phi - a * Q);
+    else if (am == ATT_15) f = n * var * ((1.f + a * a) * Q - a * phi);
+    else {  // any alpha: n E[(sd (Z - a))_+^c0] by the midpoint rule over [a, a + 8]
+      float acc = 0.f;
+      for (int i = 0; i < 32; ++i) {
+        const float x = 0.25f * ((float)i + 0.5f);
+        acc += __expf(p.c0 * __logf(sd * x)) * 0.39894228f * __expf(-0.5f * (a + x) * (a + x));
+      }
+      f = n * acc * 0.25f;
+    }
+    if (f > 1.f) lo = a;
+    else hi = a;
+  }
+  const float support = n * 0.5f * erfcf(0.5f * (lo + hi) * 0.70710678f);
+  const unsigned long long fits = __builtin_amdgcn_ballot_w64(support <= p.probe_max_support);
+  // (a spread of zero or a NaN predicts nothing: every length fits, and the kernels find out for themselves)
+  const int top = fits == 0ull ? -1 : 63 - __builtin_clzll(fits);
+  const float n_fit = top < 0 ? 0.f : (top == 63 ? INFINITY : 64.f * exp2f((float)top * (14.f / 63.f)));
   if (tid != 0) return;
-  if (dense_rows >= 3) ctrl[64 + 2 * u] = 1u << 20;  // (the sparse kernel counts the marked heads itself)
+  // A head goes one way as a whole: by its longest rows, which see all L keys and hold most of the work.  (Serving only
+  // its shorter row blocks from their supports was measured and loses: for a row block of few tiles the fixed cost of the
+  // lists outweighs the walks saved, and a launch split between the two kernels took 15 % longer than the dense kernel
+  // alone.)  A marked head: the copy of K skips it and the sparse-support kernels leave its row blocks to the dense ones.
+  const bool fits_all = n_fit >= (float)L;
+  if (p.w1_scales) p.w1_scales[4 * u + 2] = fits_all ? INFINITY : 0.f;
+  if (!fits_all) ctrl[64 + 2 * u] = 1u << 20;
 }
 
 // Workspace of the forward for the 16-bit types, for the head dims the sparse-support kernel serves: its work
@@ -213,9 +230,9 @@ static FwdWorkspace fwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     if (slots > kSparseMaxSlots) slots = kSparseMaxSlots;
     w.slots = (int)slots;
     w.queue_off = align256(w.vt_bytes);
-    // eight counters, then two hint words per K/V head and two more, then two scales per K/V head
+    // eight counters, then two hint words per K/V head and two more, then four floats per K/V head
     w.scales_off = w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8;
-    w.flags_off = align256(w.scales_off + (size_t)B * Hkv * 8);
+    w.flags_off = align256(w.scales_off + (size_t)B * Hkv * 16);
     w.events_off = align256(w.flags_off + (size_t)items * 4);
     w.k8_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
     w.total = w.k8_off + (size_t)B * Hkv * npad_of(N) * D;  // the e4m3 copy of K
@@ -247,6 +264,13 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* x, long long n)
 static bool sparse_enabled() {
   const char* e = getenv("ADSP_SPARSE");
   return !(e && strcmp(e, "0") == 0);
+}
+// The probe leaves a K/V head to the dense kernel when the support its Gaussian model predicts exceeds this many keys.
+// ADSP_PROBE_MAX_SUPPORT in the environment overrides it (0: every head is left to the dense kernel, which then runs
+// behind the sparse-support kernel as it does for the row blocks that kernel gives up; for comparisons).
+static float probe_max_support() {
+  const char* e = getenv("ADSP_PROBE_MAX_SUPPORT");
+  return e ? (float)atof(e) : 28.f;
 }
 
 // ADSP_BWD_STREAMS=0 in the environment makes the sparse-support dK/dV kernel walk for itself instead of taking the
@@ -313,6 +337,7 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   p.events = nullptr;
   p.k8 = nullptr;
   p.w1_scales = nullptr;
+  p.probe_max_support = 0.f;
   p.save_flags = nullptr;
   p.save_lens = nullptr;
   p.save_tshift = nullptr;
@@ -331,6 +356,7 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
       p.events = ws + w.events_off;
       p.k8 = ws + w.k8_off;
       p.w1_scales = (float*)(ws + w.scales_off);
+      p.probe_max_support = probe_max_support();
       if (sl.total) {
         unsigned char* sp = (unsigned char*)supports;
         p.save_flags = (int32_t*)(sp + sl.flags_off);
@@ -665,6 +691,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
       pp.c0 = p.c0;
       pp.queue = p.queue;
       pp.hints = p.hints;
+      pp.probe_max_support = probe_max_support();
       int rc;
       if (dtype == ADSP_BF16) {
         hipLaunchKernelGGL(attn_probe_kernel<bf16_t>, dim3((unsigned)(B * Hkv)), dim3(256), 0, s, pp, D, am);

@@ -83,17 +83,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
   static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
 
-  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all row blocks
-    const int units = p.B * p.Hkv;
-    int unmarked = 0;
-    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints[2 * u] < (1u << 20) ? 1 : 0;
-    if (__syncthreads_count(unmarked) == 0) {
-      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue[kCtrlAllDense] = 1u;
-      return;
-    }
+  // (the probe left too little to this kernel: the dense kernel serves everything)
+  if (sparse_steps_aside(p.hints, p.varlen, p.varlen_bits, p.B, p.Hkv, p.N)) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) p.queue[kCtrlAllDense] = 1u;
+    return;
   }
   int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
-  int known_unit = -1;   // thread 0: the K/V head whose hint counters it has last seen (or set) as served
   for (;;) {
     // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
     // of this loop they would stay live through both walks, and the walks have no registers to spare.
@@ -123,15 +118,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         int unit = got / (group * n_mblk);
         const int units = p.B * p.Hkv;
         if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
-        if (unit != known_unit) {
-          const uint32_t gave_up = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t served = __hip_atomic_load(p.hints + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
-          const uint32_t all_gave_up = __hip_atomic_load(p.hints + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t all_served = __hip_atomic_load(p.hints + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          s_skip = ((gave_up >= 3u && served == 0u) || (all_gave_up >= 64u && all_served == 0u)) ? 1 : 0;
-          if (served > 0u) known_unit = unit;
-        }
+        // (a K/V head the probe marked is left to the dense kernel; nothing else is consulted, so the same inputs take
+        // the same way on every call)
+        s_skip = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (1u << 20) ? 1 : 0;
       }
       s_giveup[0] = 0u;
       s_giveup[1] = 0u;
@@ -158,9 +147,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       L = (int)(l < 0 ? 0 : (l > N ? N : l));
     }
     int32_t* const flag = p.block_flags + ((size_t)(b * p.Hq + h) * n_mblk + mblk);
-    // Row blocks of one K/V head tend to share their fate: once a few of them were given up and none succeeded, the
-    // rest go to the dense kernel unseen (a hint only: thread 0 read the counters, without any ordering, above).
-    uint32_t* const hint = p.hints + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
     const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
     const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
     const int qi = m0 + wave * 32 + lq;
@@ -174,7 +160,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       continue;
     }
 
-    if (s_skip) {
+    // (where the forward kept its candidate stream for this row block there is no walk: see below; a row block the
+    // forward's sparse-support kernel did not serve -- its supports outgrew that kernel's lists, which are this one's --
+    // goes to the dense kernel without a walk)
+    const bool fwd_kept = p.fwd_streams != nullptr;
+    const bool from_fwd = fwd_kept && p.fwd_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] == 1;
+    if (s_skip || (fwd_kept && !from_fwd)) {
       if (tid == 0) {
         *flag = 1;
         atomicAdd(&p.queue[kCtrlFlagged], 1u);
@@ -190,8 +181,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // ---- Q fragments; rows past the valid length are zero (their scores are never used).  The forward's threshold
     // in raw score units: the walk's accumulators start at its negative, so a positive result is a member of the
     // support ----------------------------------------------------------------------------------------------------
-    // (where the forward kept its candidate stream for this row block there is no walk: see below)
-    const bool from_fwd = p.fwd_streams != nullptr && p.fwd_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] == 1;
     const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
     uint32_t qf[G::kQRegs];
 #pragma unroll
@@ -416,8 +405,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       if (tid == 0) {
         *flag = 1;
         atomicAdd(&p.queue[kCtrlFlagged], 1u);
-        atomicAdd(hint, 1u);
-        atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
       }
       continue;
     }
@@ -578,11 +565,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     }
     if (tid == 0) {
       *flag = 0;
-      if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
-        atomicAdd(hint + 1, 1u);
-        atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);
-        known_unit = b * p.Hkv + kvh;
-      }
     }
   }
 }
@@ -623,17 +605,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
   static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
 
-  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all row blocks
-    const int units = p.B * p.Hkv;
-    int unmarked = 0;
-    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints2[2 * u] < (1u << 20) ? 1 : 0;
-    if (__syncthreads_count(unmarked) == 0) {
-      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue2[kCtrlAllDense] = 1u;
-      return;
-    }
+  // (the probe left too little to this kernel: the dense kernel serves everything)
+  if (sparse_steps_aside(p.hints2, p.varlen, p.varlen_bits, p.B, p.Hkv, p.N)) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) p.queue2[kCtrlAllDense] = 1u;
+    return;
   }
   int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
-  int known_unit = -1;   // thread 0: the K/V head whose hint counters it has last seen (or set) as served
   for (;;) {
     // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
     // of this loop they would stay live through both walks, and the walks have no registers to spare.
@@ -663,19 +640,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         int unit = got / (group * n_mblk);
         const int units = p.B * p.Hkv;
         if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
-        if (unit != known_unit) {
-          const uint32_t gave_up = __hip_atomic_load(p.hints2 + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t served = __hip_atomic_load(p.hints2 + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
-          const uint32_t all_gave_up = __hip_atomic_load(p.hints2 + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t all_served = __hip_atomic_load(p.hints2 + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          // (the first key blocks of a causal sequence, which come first, collect the most queries and overflow even
-          // when the supports are short: only a long run of failures without a success says that the head is dense)
-          (void)all_gave_up;
-          (void)all_served;
-          s_skip = (gave_up >= (1u << 20) || (gave_up >= 32u && served == 0u)) ? 1 : 0;
-          if (served > 0u) known_unit = unit;
-        }
+        s_skip = __hip_atomic_load(p.hints2 + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (1u << 20) ? 1 : 0;
       }
       s_giveup[0] = 0u;
       s_giveup[1] = 0u;
@@ -703,8 +668,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     }
     // a key block that any query head gives up goes to attn_bwd_dkdv_kernel with all its heads
     int32_t* const flag = p.kv_flags + ((size_t)(b * p.Hkv + kvh) * n_mblk + mblk);
-    // the K/V head's hint counters (thread 0 read them, without any ordering, above)
-    uint32_t* const hint = p.hints2 + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
     const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
     const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
     const int qi = m0 + wave * 32 + lq;
@@ -1108,17 +1071,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       if (tid == 0) {
         *flag = 1;
         atomicAdd(&p.queue2[kCtrlFlagged], 1u);
-        atomicAdd(hint, 1u);
-        atomicAdd(p.hints2 + 2 * p.B * p.Hkv, 1u);
       }
       continue;
     }
     if (tid == 0) {
-      if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
-        atomicAdd(hint + 1, 1u);
-        atomicAdd(p.hints2 + 2 * p.B * p.Hkv + 1, 1u);
-        known_unit = b * p.Hkv + kvh;
-      }
     }
   }
 }
@@ -1157,14 +1113,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   const long long per_xcd = (total + 7) / 8;
   const float qs = p.qscale;
 
-  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all key blocks
-    const int units = p.B * p.Hkv;
-    int unmarked = 0;
-    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints2[2 * u] < (1u << 20) ? 1 : 0;
-    if (__syncthreads_count(unmarked) == 0) {
-      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue2[kCtrlAllDense] = 1u;
-      return;
-    }
+  // (the probe left too little to this kernel: the dense kernel serves everything)
+  if (sparse_steps_aside(p.hints2, p.varlen, p.varlen_bits, p.B, p.Hkv, p.N)) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) p.queue2[kCtrlAllDense] = 1u;
+    return;
   }
   int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
   for (;;) {

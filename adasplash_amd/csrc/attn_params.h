@@ -13,6 +13,7 @@ enum AttnAlphaMode { ATT_15 = 0, ATT_2 = 1, ATT_GEN = 2 };
 // control words of the sparse-support forward behind the eight work counters (AttnParams::queue)
 constexpr int kCtrlFlagged = 8;     // row blocks left to the dense kernel
 constexpr int kCtrlAllDense = 9;    // set by the sparse kernel when every K/V head was predicted dense: it served nothing
+constexpr int kCtrlGaveUp = 10;     // of the row blocks left to the dense kernel, those the sparse kernel had started on
 
 struct AttnParams {
   const void* q;
@@ -38,12 +39,16 @@ struct AttnParams {
   // 1 = left to attn_fwd_kernel, which skips the others when block_flags is set.
   int32_t* block_flags;   // [B, Hq, n_mblk], or null: attn_fwd_kernel serves every row block
   uint32_t* queue;        // eight work counters, one per XCD, then the two control words above; zero at launch
-  uint32_t* hints;        // [B * Hkv + 1][2] row blocks {given up, served} per K/V head, then over all heads; zero at launch
+  uint32_t* hints;        // [B * Hkv + 1][2]: word 0 of a K/V head is 1 << 20 when the probe leaves all of it to the dense kernel (the backward's
+                          // kernels also count row blocks {given up, served} per K/V head and over all heads here); zero at launch
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
   const unsigned char* k8;  // fp8 (e4m3) copy of K, [B * Hkv][Npad][D] bytes, rows past N zero: the operand of the first walk
-  // Powers of two per K/V head, {for q, for k}, set by the probe: q and k are multiplied by them before they are
-  // rounded for the first walk, so that its scores stay inside the range its position tags need (null: 1, 1)
+  // Four floats per K/V head, set by the probe: powers of two for q and for k (they are multiplied by them before
+  // they are rounded for the first walk, so that its scores stay inside the range its position tags need), the largest
+  // number of keys a row may see for the head's score spread to predict a support that fits the lists (infinity when the
+  // probe did not look: short sequences), and a spare word
   float* w1_scales;
+  float probe_max_support;  // the support the probe lets a row have before it leaves the row to the dense kernel
   // Supports kept for the backward (null: none kept).  The sparse-support kernel then writes its candidate streams to a
   // place of their own per (row block, wave) and leaves them there, with their lengths, every row's threshold minus
   // lower bound (raw score units: an entry is a member of the support when its value exceeds it), and a flag per row

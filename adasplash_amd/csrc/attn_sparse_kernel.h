@@ -104,6 +104,32 @@ __device__ __forceinline__ int wave_scan_i(int v) {
   return v;
 }
 
+// Should a sparse-support kernel leave the whole launch to the dense kernel?  The K/V heads the probe left unmarked
+// (`hints[2 u] < 1 << 20`) must hold at least half of the launch's work (sequence length squared), else the kernel steps
+// aside altogether: a launch split between the two kernels pays both kernels' tails, and with little to gain that
+// costs more than it saves.  Integer sums: the same decision in every workgroup and on every call.  All threads of the
+// workgroup call it together.
+__device__ __forceinline__ bool sparse_steps_aside(const uint32_t* hints, const void* varlen, int varlen_bits, int B, int Hkv, int N) {
+  __shared__ unsigned long long s_work[2];
+  if (threadIdx.x < 2) s_work[threadIdx.x] = 0ull;
+  __syncthreads();
+  const int units = B * Hkv;
+  unsigned long long mine = 0ull, all = 0ull;
+  for (int u = threadIdx.x; u < units; u += blockDim.x) {
+    long long l = N;
+    if (varlen) {
+      l = varlen_bits == 64 ? ((const long long*)varlen)[u / Hkv] : (long long)((const int*)varlen)[u / Hkv];
+      l = l < 0 ? 0 : (l > N ? N : l);
+    }
+    all += (unsigned long long)(l * l);
+    if (hints[2 * u] < (1u << 20)) mine += (unsigned long long)(l * l);
+  }
+  if (all) atomicAdd(&s_work[0], all);
+  if (mine) atomicAdd(&s_work[1], mine);
+  __syncthreads();
+  return 2ull * s_work[1] < s_work[0] || s_work[1] == 0ull;
+}
+
 template <typename T, int D> struct SparseGeo {
   using G = TileGeo<T, D>;
   static constexpr int kNW = 4;
@@ -141,7 +167,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   static_assert(AM == ATT_15 || AM == ATT_2 || AM == ATT_GEN, "alpha = 1.5, 2 or any other in (1, 2)");
   constexpr int NW = SG::kNW, BM = SG::kBM;
   __shared__ __align__(1024) unsigned char lds_all[SG::kLds];
-  __shared__ int s_item, s_skip;
+  __shared__ int s_item;
   // a lane ran out of event slots, or a wave out of list room.  Two words: the walks write the one of the tile's
   // parity and read the other one behind the next barrier, so no wave can read a word another one is still setting
   __shared__ uint32_t s_giveup[2];
@@ -161,17 +187,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
   constexpr bool kKStep = (NW * 64 / KS::kC) % 16 == 0 && (NW * 64) % KS::kC == 0;
   static_assert(kKStep && G::kKLoads % NW == 0, "head dims 32 .. 128");
 
-  {  // every K/V head marked dense by the probe: nothing to do here, the dense kernel serves all row blocks
-    const int units = p.B * p.Hkv;
-    int unmarked = 0;
-    for (int u = threadIdx.x; u < units; u += SG::kThreads) unmarked |= p.hints[2 * u] < (1u << 20) ? 1 : 0;
-    if (__syncthreads_count(unmarked) == 0) {
-      if (blockIdx.x == 0 && threadIdx.x == 0) p.queue[kCtrlAllDense] = 1u;
-      return;
-    }
+  if (sparse_steps_aside(p.hints, p.varlen, p.varlen_bits, p.B, p.Hkv, p.N)) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) p.queue[kCtrlAllDense] = 1u;
+    return;
   }
   int queues_tried = 0;  // thread 0: how many of the eight counters were found empty
-  int known_unit = -1;   // thread 0: the K/V head whose hint counters it has last seen (or set) as served
   for (;;) {
     // The lane's constants are formed anew for every row block (the empty asm hides that they repeat): hoisted out
     // of this loop they would stay live through both walks, and the walks have no registers to spare.
@@ -199,21 +219,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         ++queues_tried;
       }
       s_item = got;
-      s_skip = 0;
-      if (got >= 0) {  // the K/V head of the row block, as decoded below
-        int unit = got / (group * n_mblk);
-        const int units = p.B * p.Hkv;
-        if (units % 8 == 0) unit = (unit % (units / 8)) * 8 + unit / (units / 8);
-        if (unit != known_unit) {
-          const uint32_t gave_up = __hip_atomic_load(p.hints + 2 * unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t served = __hip_atomic_load(p.hints + 2 * unit + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          // the same over all heads, for the launches whose workgroups outnumber a head's row blocks
-          const uint32_t all_gave_up = __hip_atomic_load(p.hints + 2 * units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t all_served = __hip_atomic_load(p.hints + 2 * units + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          s_skip = ((gave_up >= 3u && served == 0u) || (all_gave_up >= 64u && all_served == 0u)) ? 1 : 0;
-          if (served > 0u) known_unit = unit;
-        }
-      }
       s_giveup[0] = 0u;
       s_giveup[1] = 0u;
     }
@@ -240,9 +245,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       L = (int)(l < 0 ? 0 : (l > N ? N : l));
     }
     int32_t* const flag = p.block_flags + ((size_t)(b * p.Hq + h) * n_mblk + mblk);
-    // Row blocks of one K/V head tend to share their fate: once a few of them were given up and none succeeded, the
-    // rest go to the dense kernel unseen (a hint only: thread 0 read the counters, without any ordering, above).
-    uint32_t* const hint = p.hints + 2 * (size_t)(b * p.Hkv + kvh);  // {given up, served}
     const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
     const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
     int32_t* const bmask_out = p.bmask ? p.bmask + ((size_t)(b * p.Hq + h) * p.n_mblk + (size_t)mblk) * p.mask_words : nullptr;
@@ -259,14 +261,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       continue;
     }
 
-    if (s_skip) {
+    const int row_hi = (m0 + BM < L ? m0 + BM : L);
+    // The probe's verdict: with this K/V head's score spread, rows that see more keys than `w1_scales[...][2]` are
+    // predicted to have supports beyond what the lists hold; such a row block goes to the dense kernel unseen.  (The
+    // same inputs take the same way on every call: nothing here depends on what other workgroups do.)
+    if ((float)(p.causal ? row_hi : L) > p.w1_scales[4 * (b * p.Hkv + kvh) + 2]) {
       if (tid == 0) {
         *flag = 1;
         atomicAdd(&p.queue[kCtrlFlagged], 1u);
       }
       continue;
     }
-    const int row_hi = (m0 + BM < L ? m0 + BM : L);
     const int nt = p.causal ? (row_hi + kBN - 1) / kBN : (L + kBN - 1) / kBN;
     const int lim = p.causal ? (qi < L - 1 ? qi : L - 1) : L - 1;
     const int wave_row0 = m0 + wave * 32;
@@ -276,7 +281,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     // values [32 lh, 32 lh + 32) of its row, in the order of the copy of K.  Rows past the valid length are zero
     // (their scores are never used). ------------------------------------------------------------------------------
     const uint16_t* const qrow = reinterpret_cast<const uint16_t*>(p.q) + qo_base + (size_t)(live ? qi : 0) * D;
-    const float aq = p.w1_scales[2 * (b * p.Hkv + kvh)], aqk = aq * p.w1_scales[2 * (b * p.Hkv + kvh) + 1];
+    const float aq = p.w1_scales[4 * (b * p.Hkv + kvh)], aqk = aq * p.w1_scales[4 * (b * p.Hkv + kvh) + 1];
     uint32_t q8[D / 64 * 8];
     uint32_t qf[G::kQRegs];  // those of the 16-bit products: loaded behind the first walk
 #pragma unroll
@@ -479,8 +484,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       if (tid == 0) {
         *flag = 1;
         atomicAdd(&p.queue[kCtrlFlagged], 1u);
-        atomicAdd(hint, 1u);
-        atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
+        atomicAdd(&p.queue[kCtrlGaveUp], 1u);
       }
       continue;
     }
@@ -755,8 +759,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       if (tid == 0) {
         *flag = 1;
         atomicAdd(&p.queue[kCtrlFlagged], 1u);
-        atomicAdd(hint, 1u);
-        atomicAdd(p.hints + 2 * p.B * p.Hkv, 1u);
+        atomicAdd(&p.queue[kCtrlGaveUp], 1u);
       }
       continue;
     }
@@ -933,11 +936,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
     if (tid == 0) {
       *flag = 0;
       if (p.save_flags) p.save_flags[(size_t)(b * p.Hq + h) * n_mblk + mblk] = 1;
-      if (known_unit != b * p.Hkv + kvh) {  // once per workgroup and K/V head is all the hints need
-        atomicAdd(hint + 1, 1u);
-        atomicAdd(p.hints + 2 * p.B * p.Hkv + 1, 1u);
-        known_unit = b * p.Hkv + kvh;
-      }
     }
   }
 }

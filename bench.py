@@ -182,6 +182,67 @@ def bench_attention(name, steps, warmup, device, backward=False):
     return res
 
 
+def bench_c4_sweep(steps, warmup, device, scales=(0.25, 0.5, 0.75, 1.0, 2.0)):
+    env_scales = os.environ.get("ADSP_BENCH_SWEEP_SCALES")
+    if env_scales:
+        scales = tuple(float(x) for x in env_scales.split(","))
+    """The headline shapes with q scaled: from flat score distributions (supports of hundreds of keys, the dense
+    kernel's case) to peaked ones (the sparse-support kernel's).  Per scale: the step as the library routes it, the step
+    with every K/V head left to the dense kernel by the probe (ADSP_PROBE_MAX_SUPPORT=0: the dense kernel as it runs
+    behind the sparse-support kernel), and the share of row blocks the sparse-support kernel served (the library's
+    control word counts the row blocks it left to the dense kernel).  The lengths and
+    the dense-equivalent FLOPs are the headline workload's."""
+    from adasplash_amd import _lib
+
+    lib = _lib.load()
+    (q0, k, v, varlen), flops, _ = make_c4(device)
+    B, Hq, N, D = q0.shape
+    Hkv = k.shape[1]
+    dt = _lib.dtype_code(q0)
+    out = torch.empty_like(q0)
+    taus = torch.empty((B, Hq, N), device=device, dtype=torch.float32)
+    bmask = torch.empty((B, Hq, lib.adsp_attn_bmask_words(N)), device=device, dtype=torch.int32)
+    nws = lib.adsp_attn_workspace_bytes(B, Hq, Hkv, N, D, dt)
+    ws = torch.zeros((nws,), device=device, dtype=torch.uint8)
+    stream = _lib.current_stream(device)
+    items = B * Hq * ((N + 127) // 128)
+    steps, warmup = max(steps, 5), max(warmup, 5)
+    points = []
+    old = os.environ.get("ADSP_PROBE_MAX_SUPPORT")
+    try:
+        for sc in scales:
+            q = (q0.float() * sc).to(q0.dtype)
+
+            def fn():
+                st = lib.adsp_attn_v2_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), taus.data_ptr(),
+                                          bmask.data_ptr(), varlen.data_ptr(), 32, B, Hq, Hkv, N, D, dt, 1,
+                                          ws.data_ptr(), nws, stream)
+                assert st == 0
+
+            os.environ.pop("ADSP_PROBE_MAX_SUPPORT", None)
+            if old is not None:
+                os.environ["ADSP_PROBE_MAX_SUPPORT"] = old
+            ms, _ = _events_ms(fn, steps, warmup)
+            # eight work counters, then {row blocks left to the dense kernel, all dense, left after work was spent on them}
+            ctrl = ws[:64].view(torch.int32).cpu()
+            left = items if int(ctrl[9]) != 0 else int(ctrl[8])
+            gave_up = 0 if int(ctrl[9]) != 0 else int(ctrl[10])
+            os.environ["ADSP_PROBE_MAX_SUPPORT"] = "0"
+            ms_dense, _ = _events_ms(fn, steps, warmup)
+            points.append({"q_scale": sc, "ms": ms, "ms_dense_kernel_only": ms_dense,
+                           "frac_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                           "row_blocks_served_by_sparse_kernel": 1.0 - left / items,
+                           "row_blocks_given_up_by_sparse_kernel": gave_up / items,
+                           "ms_over_dense_only": ms / ms_dense})
+            del q
+    finally:
+        if old is None:
+            os.environ.pop("ADSP_PROBE_MAX_SUPPORT", None)
+        else:
+            os.environ["ADSP_PROBE_MAX_SUPPORT"] = old
+    return {"steps": steps, "warmup": warmup, "points": points}
+
+
 def bench_rows(steps, warmup, device, rows=16384, cols=8192):
     """Entmax rows: rotate over several input/output pairs so every read comes from HBM, not the
     256 MB last-level cache."""
@@ -287,7 +348,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd", "c5_bwd", "c2_bwd"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c5", "c2", "copy", "c4_bwd", "c3_bwd", "c5_bwd", "c2_bwd", "c4_sweep"])
     ap.add_argument("--no-extra", action="store_true", help="skip the entmax-rows and CPU-baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -312,6 +373,14 @@ def main():
         ms, _ = _events_ms(lambda: y.copy_(x), args.steps, args.warmup)
         line.update({"value": 2 * x.numel() / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "dtype": "u8",
                      "config": {"workload": "copy: torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)"}})
+        print(json.dumps(line))
+        return
+    if args.workload == "c4_sweep":
+        sweep = bench_c4_sweep(args.steps, args.warmup, device)
+        unit = next((pt for pt in sweep["points"] if pt["q_scale"] == 1.0), sweep["points"][-1])
+        line.update({"value": unit["frac_mfma_peak"] * MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "ms_per_step": unit["ms"],
+                     "dtype": "bf16", "config": {"workload": "c4_sweep: the headline shapes with q scaled by 0.25 .. 2"},
+                     "extra": {"c4_sweep": sweep}})
         print(json.dumps(line))
         return
     if args.workload == "c2_bwd":
@@ -362,7 +431,9 @@ def main():
                     line["extra"][other]["kernel"] = FWD_KERNELS[other]
                     del r
                     torch.cuda.empty_cache()
-                b = bench_attention("c4", max(3, args.steps // 2), 1, device, backward=True)
+                line["extra"]["c4_sweep"] = bench_c4_sweep(args.steps // 2, 5, device)
+                torch.cuda.empty_cache()
+                b = bench_attention("c4", max(3, args.steps // 2), 5, device, backward=True)
                 line["extra"]["attention_backward"] = {k: b[k] for k in ("ms_per_step", "eff_tflops", "frac_mfma_peak",
                                                                          "flops_per_step")}
                 del b

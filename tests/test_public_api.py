@@ -166,7 +166,7 @@ def test_sizing_helpers_and_status_strings():
     # ... and at head dims 64 / 128 it holds that kernel's counters, flags, candidate slots (at most 1024) and copy of K
     slot = 4 * 1616 * 8
     k8 = 8 * 8 * 8192 * 128  # the one-byte copy of K
-    assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) == 256 + 1280 + 8 * 32 * 64 * 4 + 1024 * slot + k8  # (8 * 8 + 1) hint pairs and 8 * 8 scale pairs, padded to 256
+    assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) == 256 + 1792 + 8 * 32 * 64 * 4 + 1024 * slot + k8  # (8 * 8 + 1) word pairs and four floats per K/V head, padded to 256
     small = lib.adsp_attn_workspace_bytes(1, 2, 2, 128, 64, _lib.ADSP_F16)
     assert 8 * slot < small < 8 * slot + 2 * 64 * 128 * 3 + 1024
     assert lib.adsp_attn_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_F32) == 0
