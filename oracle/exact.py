@@ -204,6 +204,51 @@ def dense_entmax_attention_general(q, k, v, alpha=1.5, is_causal=False, varlen=N
     return out
 
 
+def dense_entmax_attention_general_grads(q, k, v, dout, alpha=1.5, is_causal=False, varlen=None, padding="right",
+                                         alibi_slopes=None, dtype=torch.float64):
+    """Gradients (dq, dk, dv) of ``dense_entmax_attention_general`` for the upstream gradient ``dout``: what autograd
+    returns for the example path (``examples/attention.py:34-91``; its test takes them at
+    ``tests/test_attention.py:50-77``).  Per query row, on the keys it sees: p = entmax(s), u = p^(2 - alpha),
+    dP = v_j . dout_i, dX = u * (dP - sum(u dP) / sum(u)); dq_i = sum_j dX_j k_j / sqrt(D), dk_j += dX_j q_i / sqrt(D),
+    dv_j += p_j dout_i.  The ALiBi term is a constant added to the scores and has no gradient; padded query rows and
+    the rows of ``dout`` that belong to them contribute nothing.  The same loops as the forward, so that it shares no
+    tensor expression with the implementation under test; pinned by finite differences in tests/test_oracle.py."""
+    B, H, Nq, D = q.shape
+    Nk = k.shape[2]
+    dq = torch.zeros(B, H, Nq, D, dtype=dtype)
+    dk = torch.zeros(B, H, Nk, D, dtype=dtype)
+    dv = torch.zeros(B, H, Nk, v.shape[3], dtype=dtype)
+    for b in range(B):
+        if varlen is None:
+            keys = list(range(Nk))
+        else:
+            L = int(varlen[b])
+            keys = list(range(L)) if padding == "right" else list(range(Nk - L, Nk))
+        keyset = set(keys)
+        for h in range(H):
+            for i in range(Nq):
+                if varlen is not None and Nq == Nk and i not in keyset:
+                    continue
+                pos_i = i + (Nk - Nq)
+                cols = [j for j in keys if (not is_causal) or j <= pos_i]
+                if not cols:
+                    continue
+                kc, vc = k[b, h, cols].to(dtype), v[b, h, cols].to(dtype)
+                qi, doi = q[b, h, i].to(dtype), dout[b, h, i].to(dtype)
+                s = (kc @ qi) / math.sqrt(D)
+                if alibi_slopes is not None:
+                    ref_i = (Nk - 1) if (Nq == 1 and Nk > 1) else i
+                    s = s + float(alibi_slopes[h]) * (torch.tensor(cols, dtype=dtype) - ref_i)
+                p = entmax_rows(s[None, :], alpha, dtype=dtype)[0]
+                u = torch.where(p > 0, p.clamp_min(1e-300) ** (2.0 - alpha), torch.zeros_like(p))
+                dp = vc @ doi
+                dx = u * (dp - (u * dp).sum() / u.sum())
+                dq[b, h, i] = (dx @ kc) / math.sqrt(D)
+                dk[b, h, cols] += dx[:, None] * qi[None, :] / math.sqrt(D)
+                dv[b, h, cols] += p[:, None] * doi[None, :]
+    return dq, dk, dv
+
+
 def dense_entmax_attention_grads(q, k, v, dout, alpha=1.5, is_causal=False, varlen=None, dtype=torch.float64):
     """Gradients (dq, dk, dv) of ``dense_entmax_attention`` for the upstream gradient ``dout``.
 

@@ -64,6 +64,44 @@ def test_bf16_inputs():
     _check(q, k, v, 2e-2, is_causal=False)
 
 
+@pytest.mark.parametrize("padding", ["left", "right"])
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_gradients_with_alibi_and_padding(padding, is_causal):
+    """dq, dk, dv through autograd with ALiBi slopes and a padded sequence, the reference's own case
+    (tests/test_attention.py:50-77,103-107: B=1, H=2, N=64, D=32, fp32, varlen 48, slopes 0.1 / 0.2, niter=10; its
+    bars: 1e-4 forward, 1e-3 gradients) against the loop oracle's gradients."""
+    g = torch.Generator().manual_seed(42)
+    q, k, v, do = (torch.randn(1, 2, 64, 32, generator=g) for _ in range(4))
+    varlen = torch.tensor([48], dtype=torch.int32)
+    alibi = torch.tensor([0.1, 0.2])
+    qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    out = dense.slow_entmax_attention(qg, kg, vg, varlen=varlen.to(DEV), is_causal=is_causal, padding=padding, niter=10,
+                                      alibi_slopes=alibi.to(DEV))
+    dq, dk, dv = torch.autograd.grad(out, (qg, kg, vg), do.to(DEV))
+    want = exact.dense_entmax_attention_general(q, k, v, 1.5, is_causal, varlen=varlen, padding=padding, alibi_slopes=alibi)
+    wq, wk, wv = exact.dense_entmax_attention_general_grads(q, k, v, do, 1.5, is_causal, varlen=varlen, padding=padding,
+                                                            alibi_slopes=alibi)
+    assert (out.double().cpu() - want).abs().max().item() < 1e-4
+    for name, got, w in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+        assert (got.double().cpu() - w).abs().max().item() < 1e-3, name
+    dead = slice(48, None) if padding == "right" else slice(0, 16)
+    assert (dq[0, :, dead] == 0).all() and (dk[0, :, dead] == 0).all() and (dv[0, :, dead] == 0).all()
+
+
+def test_gradients_with_fewer_queries_than_keys():
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(2, 2, 5, 16, generator=g)
+    k, v = (torch.randn(2, 2, 33, 16, generator=g) for _ in range(2))
+    do = torch.randn(2, 2, 5, 16, generator=g)
+    slopes = torch.tensor([0.5, 0.1])
+    qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    out = dense.slow_entmax_attention(qg, kg, vg, is_causal=True, niter=10, alibi_slopes=slopes.to(DEV))
+    got = torch.autograd.grad(out, (qg, kg, vg), do.to(DEV))
+    want = exact.dense_entmax_attention_general_grads(q, k, v, do, 1.5, True, alibi_slopes=slopes)
+    for name, a, w in zip(("dq", "dk", "dv"), got, want):
+        assert (a.double().cpu() - w).abs().max().item() < 1e-3, name
+
+
 def test_argument_errors():
     q, k, v = (t.to(DEV) for t in _qkv(2, 2, 8, 8, 16, torch.float32))
     with pytest.raises(ValueError):

@@ -214,6 +214,60 @@ def test_closed_form_gradients_match_finite_differences(alpha, causal, shape, va
 
 
 # ---- the dense example path with ALiBi, left padding and q_len != k_len (examples/attention.py:8-91) ----------
+@pytest.mark.parametrize("alpha", [1.5, 2.0, 1.333])
+@pytest.mark.parametrize("causal,padding,nq,varlen", [
+    (True, "right", 7, [7, 4]), (False, "left", 7, [5, 7]), (True, "left", 7, [3, 6]), (True, "right", 3, None),
+    (False, "right", 1, [7, 2]),
+])
+def test_general_path_gradients_match_finite_differences(alpha, causal, padding, nq, varlen):
+    # pins dense_entmax_attention_general_grads (ALiBi, both padding sides, fewer queries than keys): central
+    # differences of the general forward oracle in fp64 along random directions of (q, k, v) -- a wrong term in any of
+    # the three gradients shows in every direction -- and, for one case, along every coordinate
+    B, H, Nk, D = 2, 2, 7, 3
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn(B, H, nq, D, generator=g, dtype=torch.float64)
+    k = torch.randn(B, H, Nk, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, H, Nk, D, generator=g, dtype=torch.float64)
+    do = torch.randn(B, H, nq, D, generator=g, dtype=torch.float64)
+    vl = torch.tensor(varlen) if varlen is not None else None
+    slopes = torch.tensor([0.3, 0.05], dtype=torch.float64)
+    kw = dict(alpha=alpha, is_causal=causal, varlen=vl, padding=padding, alibi_slopes=slopes)
+    grads = exact.dense_entmax_attention_general_grads(q, k, v, do, **kw)
+
+    def loss(qq, kk, vv):
+        return (exact.dense_entmax_attention_general(qq, kk, vv, **kw) * do).sum().item()
+
+    eps = 1e-6
+    every_coordinate = alpha == 1.5 and causal and padding == "left"
+    dirs = []
+    if every_coordinate:
+        for which, t in enumerate((q, k, v)):
+            for i in range(t.numel()):
+                d = [torch.zeros_like(x) for x in (q, k, v)]
+                d[which].view(-1)[i] = 1.0
+                dirs.append(d)
+    else:
+        for which in range(6):  # two directions in each of q, k, v alone, so that no two gradients can trade errors
+            d = [torch.zeros_like(x) for x in (q, k, v)]
+            d[which % 3] = torch.randn(d[which % 3].shape, generator=g, dtype=torch.float64)
+            dirs.append(d)
+    for dq_, dk_, dv_ in dirs:
+        num = (loss(q + eps * dq_, k + eps * dk_, v + eps * dv_) - loss(q - eps * dq_, k - eps * dk_, v - eps * dv_)) / (2 * eps)
+        ana = (grads[0] * dq_).sum().item() + (grads[1] * dk_).sum().item() + (grads[2] * dv_).sum().item()
+        assert abs(num - ana) < 1e-7 * max(1.0, abs(ana))
+
+
+def test_general_path_gradients_reduce_to_the_plain_ones():
+    # without ALiBi, right padded, q_len == k_len: the closed form over whole tensors must agree with the loops
+    g = torch.Generator().manual_seed(19)
+    q, k, v, do = (torch.randn(2, 2, 9, 4, generator=g, dtype=torch.float64) for _ in range(4))
+    vl = torch.tensor([9, 5])
+    a = exact.dense_entmax_attention_general_grads(q, k, v, do, 1.5, True, vl)
+    b = exact.dense_entmax_attention_grads(q, k, v, do, 1.5, True, vl)
+    for x, y in zip(a, b):
+        assert (x - y).abs().max() < 1e-12
+
+
 
 def _rand_qkv(B, H, Nq, Nk, D, seed=0):
     g = torch.Generator().manual_seed(seed)
