@@ -75,6 +75,15 @@ def triton_entmax15(x, **kwargs):
     return triton_entmax15(x, **kwargs)
 
 
+def set_keep_supports(mode):
+    """What the attention forward keeps for its backward besides the reference's saved tensors: ``"auto"`` (the supports
+    it found, when they take at most twice the bytes of q or 256 MiB), ``"always"`` or ``"never"`` (the backward then
+    finds the supports again with a score walk).  Returns the previous mode.  Not part of the reference's surface."""
+    from ._attention import set_keep_supports as _set
+
+    return _set(mode)
+
+
 adasplash2 = _adasplash_v2
 
 __all__ = [

@@ -15,18 +15,49 @@ def _varlen_bits(varlen):
     raise AssertionError(f"varlen must be int32/int64; got {varlen.dtype}.")
 
 
-def keep_supports_enabled():
-    """``ADSP_KEEP_SUPPORTS=0`` in the environment: the forward keeps nothing for the backward (comparisons, tests, or to
-    save the memory: 51 KB per 128 query rows and head)."""
-    import os
-    return os.environ.get("ADSP_KEEP_SUPPORTS", "1") != "0"
+# What the forward of the autograd functions keeps for the backward besides q, k, v, taus and bmask: the supports it
+# found (51.7 KB per 128 query rows and head, whatever the head dim), with which the backward needs no score walk of
+# its own.  "auto" keeps them when they take at most twice the bytes of q -- the reference keeps a second output of
+# q's size for its backward (adasplash/adasplash_v2.py:1421-1426) -- or 256 MiB; "always" and "never" say what they
+# mean.  ``ADSP_KEEP_SUPPORTS`` in the environment sets the initial mode (0 / never, 1 / always, auto).
+_KEEP_MODES = ("auto", "always", "never")
+_keep_mode = None
+
+
+def set_keep_supports(mode):
+    """Choose what the attention forward keeps for its backward: ``"auto"`` (default), ``"always"`` or ``"never"``.
+    Returns the previous mode."""
+    global _keep_mode
+    if mode not in _KEEP_MODES:
+        raise ValueError(f"mode must be one of {_KEEP_MODES}; got {mode!r}")
+    old = get_keep_supports()
+    _keep_mode = mode
+    return old
+
+
+def get_keep_supports():
+    global _keep_mode
+    if _keep_mode is None:
+        import os
+
+        env = os.environ.get("ADSP_KEEP_SUPPORTS", "auto").lower()
+        _keep_mode = {"0": "never", "1": "always"}.get(env, env if env in _KEEP_MODES else "auto")
+    return _keep_mode
+
+
+def _keeps(sup_bytes, q):
+    mode = get_keep_supports()
+    if mode == "never" or sup_bytes == 0:
+        return False
+    return mode == "always" or sup_bytes <= max(2 * q.numel() * q.element_size(), 256 << 20)
 
 
 def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_counts=None, keep_supports=False):
     """Allocate out / taus / bmask / workspace with torch and enqueue the fused forward on the
     current stream.  Returns ``(out, taus, bmask)``, and with ``keep_supports`` a fourth value: the buffer in which the
     forward keeps the supports it found for ``launch_backward`` (``None`` where the library keeps none: fp32, head dims
-    other than 64 / 128, a caller that asks for the tile statistics)."""
+    other than 64 / 128, a caller that asks for the tile statistics, or a buffer beyond what ``set_keep_supports``
+    allows; ``keep_supports="always"`` asks for the buffer whatever the mode)."""
     _lib.require_device(q, k, v, varlen)
     lib = _lib.load()
     B, Hq, N, D = q.shape
@@ -40,10 +71,10 @@ def launch_forward(q, k, v, *, version, alpha, is_causal, niter, varlen, tile_co
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
     bits = _varlen_bits(varlen)
     sup = None
-    if keep_supports and tile_counts is None and keep_supports_enabled():
+    if keep_supports and tile_counts is None:
         sup_bytes = lib.adsp_attn_supports_bytes(B, Hq, Hkv, N, D, dt)
-        if sup_bytes:
-            sup = torch.empty((sup_bytes,), device=q.device, dtype=torch.uint8)
+        if keep_supports == "always" or _keeps(sup_bytes, q):  # ("always": a caller that asks for them by name)
+            sup = torch.empty((sup_bytes,), device=q.device, dtype=torch.uint8) if sup_bytes else None
     with _lib.device_guard(q.device):
         stream = _lib.current_stream(q.device)
         if sup is not None and version == 2:

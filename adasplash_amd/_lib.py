@@ -21,6 +21,7 @@ _vp, _i, _i64, _sz, _dbl = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes
 _SIGNATURES = {
     "adsp_version": (_i, []),
     "adsp_build_id": (ctypes.c_char_p, []),
+    "adsp_build_flags": (ctypes.c_char_p, []),
     "adsp_status_string": (ctypes.c_char_p, [_i]),
     "adsp_entmax_rows_fwd": (_i, [_vp, _vp, _i64, _i64, _i, _dbl, _i, _i, _i, _vp]),
     "adsp_entmax_rows_bwd": (_i, [_vp, _vp, _vp, _i64, _i64, _i, _dbl, _vp]),
@@ -79,7 +80,9 @@ def _check_build_id(lib):
 
     if not _build.CSRC.is_dir() or not _build.INCLUDE.is_dir():
         return
-    have, want = lib.adsp_build_id().decode(), _build.source_id()
+    # (the id covers the extra flags of the build, which the library names itself: the environment of this process,
+    # which may differ from the build's, does not enter)
+    have, want = lib.adsp_build_id().decode(), _build.source_id(lib.adsp_build_flags().decode())
     if have != want:
         raise RuntimeError(
             f"{_LIB_PATH} is stale: it was built from sources with id {have}, the tree has id {want}. "

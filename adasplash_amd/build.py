@@ -5,9 +5,11 @@ linked into ``adasplash_amd/lib/libadasplash_hip.so`` (the C ABI declared in ``i
 
 * An object is recompiled when the hash of its command line, its source and every header it includes
   (transitively, quoted includes) differs from the one recorded beside it; ``--force`` recompiles everything.
-* The library carries ``adsp_build_id()``: a hash over all kernel sources, headers and flags.  ``source_id()``
-  recomputes it from the tree, and the loader and the tests compare the two, so a library that is older than
-  the sources next to it is an error instead of a silent stale binary.
+* The library carries ``adsp_build_id()``: a hash over all kernel sources, headers and flags, and
+  ``adsp_build_flags()``: the extra flags it was built with (``ADSP_ATTN_FLAGS`` in the environment of the build:
+  profiling builds).  ``source_id(extra)`` recomputes the id from the tree for the library's own extra flags, and the
+  loader and the tests compare the two, so a library that is older than the sources next to it is an error instead
+  of a silent stale binary, whatever the environment of the process that loads it.
 * The link step always runs, and the library is replaced atomically after a successful link only.
 """
 
@@ -38,24 +40,27 @@ FLAGS = [
 ]
 # The attention kernels never produce or consume NaNs on purpose (masked scores are -inf and are clamped
 # before any product), so fmax/fmin need no sNaN-quieting pre-pass there.
-ATTN_FLAGS = ["-fno-honor-nans"] + os.environ.get("ADSP_ATTN_FLAGS", "").split()
+ATTN_FLAGS = ["-fno-honor-nans"]
+EXTRA_ATTN_FLAGS = os.environ.get("ADSP_ATTN_FLAGS", "").split()  # of this process: what a build started here adds
 
 TYPES = {"f32": "float", "bf16": "bf16_t", "f16": "f16_t"}
 HEAD_DIMS = (16, 32, 64, 128, 256)
 
 
-def units():
-    """(object stem, source file, extra flags) of every translation unit."""
+def units(extra=None):
+    """(object stem, source file, extra flags) of every translation unit; ``extra``: flags added to the attention units
+    (default: ``ADSP_ATTN_FLAGS`` of this process)."""
+    attn_flags = ATTN_FLAGS + (EXTRA_ATTN_FLAGS if extra is None else list(extra))
     out = [("attn_api", "attn_api.hip", []), ("entmax_rows", "entmax_rows.hip", [])]
     for tag, ty in TYPES.items():
         for d in HEAD_DIMS:
             base = [f"-DADSP_T={ty}", f"-DADSP_TAG={tag}", f"-DADSP_D={d}"]
             for multi in (0, 1):
-                out.append((f"attn_fwd_{tag}_d{d}_m{multi}", "attn_fwd_unit.hip", base + [f"-DADSP_MULTI={multi}"] + ATTN_FLAGS))
+                out.append((f"attn_fwd_{tag}_d{d}_m{multi}", "attn_fwd_unit.hip", base + [f"-DADSP_MULTI={multi}"] + attn_flags))
             out.append((f"attn_bwd_{tag}_d{d}", "attn_bwd_unit.hip", base))
             if tag != "f32" and d in (64, 128):
-                out.append((f"attn_sparse_{tag}_d{d}", "attn_sparse_unit.hip", base + ATTN_FLAGS))
-                out.append((f"attn_bwd_sparse_{tag}_d{d}", "attn_bwd_sparse_unit.hip", base + ATTN_FLAGS))
+                out.append((f"attn_sparse_{tag}_d{d}", "attn_sparse_unit.hip", base + attn_flags))
+                out.append((f"attn_bwd_sparse_{tag}_d{d}", "attn_bwd_sparse_unit.hip", base + attn_flags))
     return out
 
 
@@ -83,13 +88,16 @@ def _digest(parts) -> str:
     return h.hexdigest()
 
 
-def source_id() -> str:
-    """Hash of everything the library is built from; what ``adsp_build_id()`` of an up-to-date library returns."""
+def source_id(extra=None) -> str:
+    """Hash of everything the library is built from; what ``adsp_build_id()`` of an up-to-date library returns.
+    ``extra``: the extra attention flags to assume (a string or a list; default: those of this process)."""
+    if isinstance(extra, str):
+        extra = extra.split()
     files = sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h")))
     parts = []
     for f in files:
         parts += [f.name, f.read_bytes()]
-    parts += FLAGS + ["--"] + ATTN_FLAGS + ["--"] + [u[0] + " " + " ".join(u[2]) for u in units()]
+    parts += FLAGS + ["--"] + [u[0] + " " + " ".join(u[2]) for u in units(extra)]
     return _digest(parts)[:16]
 
 
@@ -101,6 +109,7 @@ def _compile(unit, build_id: str, force: bool):
     extra = list(extra)
     if stem == "attn_api":
         extra.append(f'-DADSP_BUILD_ID="{build_id}"')
+        extra.append('-DADSP_BUILD_FLAGS="' + " ".join(EXTRA_ATTN_FLAGS).replace('"', "") + '"')
     cmd = [HIPCC, *FLAGS, *extra, "-c", str(src_path), "-o", str(obj)]
     deps = _deps(src_path)
     sig = _digest([" ".join(cmd)] + [x for p in sorted(deps) for x in (str(p), deps[p])])

@@ -321,8 +321,8 @@ static int attn_common(const void* q, const void* k, const void* v, void* out, f
   // Sparse-support kernel first (16-bit types, alpha 1.5 / 2 or any other in [1.125, 2): below that its solver on the
   // lists would need too many rounds; either entry point, no tile statistics asked for): it serves the row blocks
   // whose supports are short and flags the others for the dense kernel.
-  const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2 || (alpha >= 1.125 && alpha < 2.0)) && !tile_counts &&
-                      (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
+  const bool sparse = w.slots > 0 && (am == ATT_15 || am == ATT_2 || (alpha >= 1.125 && alpha < 2.0)) &&
+                      !tile_counts && (long long)B * Hq * mblocks_of(N) < (1ll << 31) && sparse_enabled();
   if (!sparse) niter += 1;
   p.niter = niter;
   p.causal = is_causal ? 1 : 0;
@@ -509,7 +509,8 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     w.queue2_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
     w.kvflags_off = align256(w.queue2_off + 256 + ((size_t)B * Hkv + 1) * 8);
     w.part_off = align256(w.kvflags_off + (size_t)B * Hkv * mblocks_of(N) * 4);
-    w.part_bytes = (size_t)B * Hq * N * D * 4;
+    // (with one query head per K/V head the kernel on the streams writes dK and dV itself: no partial rows)
+    w.part_bytes = (Hq == Hkv && bwd_streams_enabled()) ? 0 : (size_t)B * Hq * N * D * 4;
     // the dQ kernel's streams, kept per (row block, wave) for the dK/dV kernel, and where their 32-key blocks start
     w.streams_off = align256(w.part_off + 2 * w.part_bytes);
     w.dir_stride = (mblocks_of(N) * 4 + 2) / 2 * 2;
@@ -770,6 +771,10 @@ extern "C" int adsp_version(void) { return 3; }
 #define ADSP_BUILD_ID "unknown"
 #endif
 extern "C" const char* adsp_build_id(void) { return ADSP_BUILD_ID; }
+#ifndef ADSP_BUILD_FLAGS
+#define ADSP_BUILD_FLAGS ""
+#endif
+extern "C" const char* adsp_build_flags(void) { return ADSP_BUILD_FLAGS; }
 
 extern "C" const char* adsp_status_string(int status) {
   switch (status) {

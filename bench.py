@@ -158,6 +158,7 @@ def bench_attention(name, steps, warmup, device, backward=False):
             kw = dict(alpha=1.5, is_causal=True)
             fwd_kw = dict(version=2, niter=1, **kw)
         out, taus, bmask, supports = _attention.launch_forward(q, k, v, varlen=varlen, keep_supports=True, **fwd_kw)
+        cfg = dict(cfg, supports_kept_bytes=0 if supports is None else supports.numel())
         dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(7)).to(q.dtype).to(device)
         fn = lambda: _attention.launch_backward(q, k, v, dout, taus, bmask, varlen=varlen,  # noqa: E731
                                                 supports=supports, **kw)
@@ -169,7 +170,19 @@ def bench_attention(name, steps, warmup, device, backward=False):
     ms, wall_ms = _events_ms(fn, steps, warmup)
     tflops = flops / (ms * 1e-3) / 1e12
     res = {"ms_per_step": ms, "wall_ms_per_step": wall_ms, "eff_tflops": tflops, "flops_per_step": flops,
-           "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS, "config": cfg}
+           "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS, "config": cfg, "steps": steps, "warmup": warmup}
+    if name == "c4" and not backward:
+        # the same forward as the autograd function runs it when a gradient is asked for: it also keeps the supports
+        # it found for the backward (its candidate streams go to a buffer of their own instead of the workspace)
+        from adasplash_amd import _attention
+
+        keep_fn = lambda: _attention.launch_forward(q, k, v, version=2, alpha=1.5, is_causal=True, niter=1,  # noqa: E731
+                                                    varlen=varlen, keep_supports="always")
+        kms, _ = _events_ms(keep_fn, steps, warmup)
+        kept = keep_fn()[3]
+        res["forward_keeping_supports"] = {"ms_per_step": kms, "supports_bytes": 0 if kept is None else kept.numel(),
+                                           "steps": steps, "warmup": warmup}
+        del kept
     if name in ("c4", "c3") and not backward:
         res["tiles"] = v2_tile_stats(q, k, v, varlen)
     if name == "c5" and not backward:
@@ -274,7 +287,7 @@ def bench_rows(steps, warmup, device, rows=16384, cols=8192):
             ms, _ = _events_ms(fn, max(steps, 100), max(warmup, 200))
             gbs = nbytes / (ms * 1e-3) / 1e9
             out[f"{dname}_alpha{alpha}"] = {"ms": ms, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
-                                            "bytes": nbytes}
+                                            "bytes": nbytes, "steps": max(steps, 100), "warmup": max(warmup, 200)}
         del xs, ys
         torch.cuda.empty_cache()
     return out
@@ -310,7 +323,8 @@ def bench_rows_backward(steps, warmup, device, rows=16384, cols=8192):
 
         ms, _ = _events_ms(fn, max(steps, 100), max(warmup, 200))
         gbs = nbytes / (ms * 1e-3) / 1e9
-        out[f"{dname}_alpha1.5"] = {"ms": ms, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS, "bytes": nbytes}
+        out[f"{dname}_alpha1.5"] = {"ms": ms, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS, "bytes": nbytes,
+                                    "steps": max(steps, 100), "warmup": max(warmup, 200)}
         del ys, dys, dxs
         torch.cuda.empty_cache()
     return out
@@ -411,7 +425,7 @@ def main():
                                   "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
                                   "kernel": BWD_KERNELS[args.workload] if bwd else FWD_KERNELS[args.workload],
                                   "flops_per_launch": res["flops_per_step"]},
-                     "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k == "wall_ms_per_step"}})
+                     "extra": {k: v for k, v in res.items() if k.startswith("tiles") or k in ("wall_ms_per_step", "forward_keeping_supports")}})
         if bwd and args.workload != "c3_bwd":
             # with the supports kept the sparse kernels issue no matrix products at all: the dense-equivalent rate
             # says how fast a dense implementation would have to be, and may exceed the matrix pipe's peak
@@ -435,7 +449,8 @@ def main():
                 torch.cuda.empty_cache()
                 b = bench_attention("c4", max(3, args.steps // 2), 5, device, backward=True)
                 line["extra"]["attention_backward"] = {k: b[k] for k in ("ms_per_step", "eff_tflops", "frac_mfma_peak",
-                                                                         "flops_per_step")}
+                                                                         "flops_per_step", "steps", "warmup")}
+                line["extra"]["attention_backward"]["supports_kept_bytes"] = b["config"]["supports_kept_bytes"]
                 del b
                 torch.cuda.empty_cache()
     if not args.no_extra:

@@ -57,6 +57,8 @@ int adsp_version(void);
  * it with the tree it sits in so that a library older than its sources cannot be tested or benchmarked.
  */
 const char* adsp_build_id(void);
+/* The extra compiler flags of a profiling build (empty for a regular one); they enter adsp_build_id(). */
+const char* adsp_build_flags(void);
 
 /* Static, NUL-terminated description of a status code. */
 const char* adsp_status_string(int status);

@@ -220,25 +220,27 @@ def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B
 ])
 def test_backward_with_and_without_the_supports_the_forward_kept(alpha, causal, B, Hq, Hkv, N, D, dtype, lens, version, scale, sparse):
     """With a gradient asked for the forward keeps the supports it found and the dQ kernel takes them from there
-    (default); ADSP_KEEP_SUPPORTS=0 makes it find them again with its score walk.  Both must meet the oracle and agree
-    with each other (the same members up to scores that differ by a rounding)."""
+    (``set_keep_supports("always")``; "auto" does the same up to a size); "never" makes it find them again with its
+    score walk.  Both must meet the oracle and agree with each other (the same members up to scores that differ by a
+    rounding)."""
     import os
     varlen = None if lens is None else torch.tensor(lens, dtype=torch.int32)
-    old = {k: os.environ.get(k) for k in ("ADSP_KEEP_SUPPORTS", "ADSP_SPARSE")}
+    old = os.environ.get("ADSP_SPARSE")
+    old_mode = A.set_keep_supports("always")
     got = {}
     try:
         os.environ["ADSP_SPARSE"] = sparse
-        for mode in ("1", "0"):
-            os.environ["ADSP_KEEP_SUPPORTS"] = mode
+        for mode in ("always", "never"):
+            A.set_keep_supports(mode)
             got[mode], want = run_case(alpha, causal, B, Hq, Hkv, N, D, dtype, varlen=varlen, version=version, seed=6, scale=scale)
             check(got[mode], want, dtype)
     finally:
-        for k, v in old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
-    for a, b in zip(got["1"], got["0"]):
+        A.set_keep_supports(old_mode)
+        if old is None:
+            os.environ.pop("ADSP_SPARSE", None)
+        else:
+            os.environ["ADSP_SPARSE"] = old
+    for a, b in zip(got["always"], got["never"]):
         assert max_err(a, b.float().cpu(), report=False) < 1.6e-2  # (a unit in the last place of a bf16 value in [1, 2) is 7.8e-3)
 
 

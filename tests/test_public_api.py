@@ -154,7 +154,10 @@ def test_library_is_built_from_the_sources_in_the_tree():
     lib.adsp_build_id.restype = ctypes.c_char_p
     have = lib.adsp_build_id().decode()
     assert re.fullmatch(r"[0-9a-f]{16}", have), have
-    assert have == build.source_id(), "libadasplash_hip.so is stale: run `python -m adasplash_amd.build`"
+    lib.adsp_build_flags.restype = ctypes.c_char_p
+    flags = lib.adsp_build_flags().decode()  # the extra flags of a profiling build (empty otherwise) enter the id
+    assert have == build.source_id(flags), "libadasplash_hip.so is stale: run `python -m adasplash_amd.build`"
+    assert build.source_id("-DADSP_SPARSE_STOP=1") != build.source_id("")
     assert _lib.build_id() == have  # and the loader, which makes the same comparison, accepts it
 
 
@@ -211,3 +214,27 @@ def test_dense_example_names_and_signatures():
     sig = inspect.signature(dense.flash_entmax_attention)
     assert list(sig.parameters) == ["q", "k", "v", "alpha", "varlen", "is_causal", "niter"]
     assert sig.parameters["is_causal"].default is True
+
+
+def test_keep_supports_modes():
+    """What the forward keeps for the backward is a mode of the package, not an environment variable only."""
+    import torch
+
+    import adasplash_amd
+    from adasplash_amd import _attention
+
+    old = adasplash_amd.set_keep_supports("never")
+    try:
+        assert old in ("auto", "always", "never")
+        q = torch.zeros(1, 2, 1024, 64, dtype=torch.bfloat16)  # 256 KB
+        assert not _attention._keeps(1 << 20, q)
+        adasplash_amd.set_keep_supports("always")
+        assert _attention._keeps(1 << 40, q) and not _attention._keeps(0, q)
+        adasplash_amd.set_keep_supports("auto")
+        assert _attention._keeps(256 << 20, q) and not _attention._keeps((256 << 20) + 1, q)
+        big = torch.zeros(1, 1, 1, 1, dtype=torch.bfloat16).expand(8, 32, 8192, 128)  # the headline q: 512 MiB
+        assert _attention._keeps(860 << 20, big) and not _attention._keeps(1100 << 20, big)
+        with pytest.raises(ValueError):
+            adasplash_amd.set_keep_supports("sometimes")
+    finally:
+        adasplash_amd.set_keep_supports(old)
