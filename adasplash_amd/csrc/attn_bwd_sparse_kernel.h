@@ -26,7 +26,7 @@ __device__ __forceinline__ void dma4s(const void* gbase, uint32_t off, void* lds
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
                :
                : "v"(off), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(base))
-               : "memory");
+               : "memory", "m0");
 }
 
 // sum over a group of LANES (8 or 16) adjacent lanes, left in every lane of the group

@@ -3,8 +3,21 @@
  *
  * Every entry point takes raw device pointers, sizes and scalars, enqueues its kernels on the
  * HIP stream it is given (a hipStream_t passed as void*; NULL = the default stream), never
- * synchronises, never allocates and keeps no state between calls.  The caller owns every buffer,
- * including the workspace.  The return value is an adsp_status; nothing is thrown across the ABI.
+ * synchronises and never allocates.  The caller owns every buffer, including the workspace; what a call
+ * computes depends on its arguments alone.  The return value is an adsp_status; nothing is thrown across
+ * the ABI.
+ *
+ * State the library does hold, none of which carries results from one call to the next:
+ *   - per process, the number of workgroups of the persistent kernels that fit the device, looked up on
+ *     the first launch of each kernel (one device family per process is assumed: gfx950);
+ *   - per device, the address of the 64 MiB scratch array behind adsp_attn_v2_fwd_noalloc, looked up on
+ *     that entry point's first call on the device (calls through it share the array: see there);
+ *   - the environment, read on every call (comparisons, tests and profiling; unset in normal use):
+ *       ADSP_SPARSE=0               every row block on the dense kernels (no sparse-support kernels)
+ *       ADSP_BWD_STREAMS=0          the sparse-support dK/dV kernel walks the scores itself instead of taking
+ *                                   the dQ kernel's candidate streams
+ *       ADSP_PROBE_MAX_SUPPORT=n    the support the probe lets a K/V head's longest rows have before it
+ *                                   leaves the head to the dense kernels (default 28; 0: every head)
  *
  * The entry points replace the Triton launches inside the reference's autograd wrappers (the
  * reference has no FFI of its own; these are the calls a binding would make in their place):
