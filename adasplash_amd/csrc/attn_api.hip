@@ -487,7 +487,7 @@ namespace adsp {
 // counters, per-row-block flags and candidate streams (the forward's layout without the copy of K).  (The dense
 // kernels need none: they read k, q and dout row-major and transpose in the LDS read.)
 struct BwdWorkspace {
-  size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, part_off, part_bytes, streams_off, dir_off, total;
+  size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, scratch_off, part_off, part_bytes, streams_off, dir_off, total;
   int slots;       // 0: no sparse-support kernels for these dimensions
   int dir_stride;  // offsets per stream of the hand-over table
 };
@@ -508,7 +508,9 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     // partial rows of dK and dV per query head
     w.queue2_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
     w.kvflags_off = align256(w.queue2_off + 256 + ((size_t)B * Hkv + 1) * 8);
-    w.part_off = align256(w.kvflags_off + (size_t)B * Hkv * mblocks_of(N) * 4);
+    // (fp32 sums of an item worked off in parts: 32 rows of dK | dV per wave of every workgroup)
+    w.scratch_off = align256(w.kvflags_off + (size_t)B * Hkv * mblocks_of(N) * 4);
+    w.part_off = align256(w.scratch_off + (size_t)slots * 4 * 32 * 2 * D * 4);
     // (with one query head per K/V head the kernel on the streams writes dK and dV itself: no partial rows)
     w.part_bytes = (Hq == Hkv && bwd_streams_enabled()) ? 0 : (size_t)B * Hq * N * D * 4;
     // the dQ kernel's streams, kept per (row block, wave) for the dK/dV kernel, and where their 32-key blocks start
@@ -535,9 +537,9 @@ __global__ __launch_bounds__(256) void bwd_ctrl_clear_kernel(uint32_t* ctrl2, co
 }
 
 // dK, dV = sum over the query heads of a K/V head of the sparse-support kernel's fp32 partial rows; key blocks left to
-// attn_bwd_dkdv_kernel are skipped (that kernel writes them).  A thread adds up 8 columns of one key row.  Rows past
-// the valid length are zeros and their partial rows are not read (the key blocks that lie wholly in the padding have
-// none).
+// attn_bwd_dkdv_kernel are skipped (that kernel writes them).  A thread adds up 8 columns of
+// one key row.  Rows past the valid length are zeros and their partial rows are not read (the key blocks that lie
+// wholly in the padding have none).
 typedef float reduce_f32x4 __attribute__((ext_vector_type(4)));
 template <typename T>
 __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restrict__ dk_part, const float* __restrict__ dv_part,
@@ -562,8 +564,10 @@ __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restric
   for (int i = 0; i < 8; ++i) sk[i] = sv[i] = 0.f;
   for (int g = 0; g < (row < L ? group : 0); ++g) {
     const size_t at = (((size_t)(b * Hq + kvh * group + g) * N) + row) * D + c * 8;
-    const reduce_f32x4 k0 = *reinterpret_cast<const reduce_f32x4*>(dk_part + at), k1 = *reinterpret_cast<const reduce_f32x4*>(dk_part + at + 4);
-    const reduce_f32x4 v0 = *reinterpret_cast<const reduce_f32x4*>(dv_part + at), v1 = *reinterpret_cast<const reduce_f32x4*>(dv_part + at + 4);
+    const reduce_f32x4 k0 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dk_part + at));
+    const reduce_f32x4 k1 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dk_part + at + 4));
+    const reduce_f32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dv_part + at));
+    const reduce_f32x4 v1 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dv_part + at + 4));
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       sk[i] += k0[i];
@@ -636,6 +640,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   p.kv_flags = nullptr;
   p.dk_part = nullptr;
   p.dv_part = nullptr;
+  p.part_scratch = nullptr;
   p.streams = nullptr;
   p.stream_dir = nullptr;
   p.dir_stride = 0;
@@ -717,6 +722,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
     p.queue2 = (uint32_t*)(ws + w.queue2_off);
     p.hints2 = p.queue2 + 64;
     p.kv_flags = (int32_t*)(ws + w.kvflags_off);
+    p.part_scratch = (float*)(ws + w.scratch_off);
     if (w.part_bytes) {
       p.dk_part = (float*)(ws + w.part_off);
       p.dv_part = (float*)(ws + w.part_off + w.part_bytes);

@@ -24,13 +24,15 @@ struct AttnBwdParams {
   uint32_t* queue;        // control words: work counters, flagged count, "every head dense"
   uint32_t* hints;        // two counters per K/V head and one pair over all heads
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
-  // the sparse-support dK/dV kernel: a control block of its own, one flag per (K/V head, key block), and fp32 partial
-  // rows [B, Hq, N, D] when a K/V head serves several query heads (null otherwise); the streams are shared
+  // the sparse-support dK/dV kernel: a control block of its own, one flag per (K/V head, key block), fp32 partial rows
+  // [B, Hq, N, D] when a K/V head serves several query heads (null otherwise), and per workgroup and wave 32 fp32
+  // rows of dK | dV for the sums of an item that is worked off in parts; the streams are shared
   uint32_t* queue2;
   uint32_t* hints2;
   int32_t* kv_flags;  // [B, Hkv, n_mblk] 1 = key block left to attn_bwd_dkdv_kernel
   float* dk_part;
   float* dv_part;
+  float* part_scratch;  // [slots, waves, 32, 2 D]
   // hand-over of the supports from the dQ kernel to the dK/dV kernel (null: the dK/dV kernel walks for itself): the dQ
   // kernel's streams kept per (row block, wave) instead of per workgroup, and per stream the offsets of the 32-key blocks
   unsigned char* streams;  // [B, Hq, n_mblk, waves, stream capacity] (score - threshold, key | row << 20) pairs

@@ -9,13 +9,38 @@
 // with u = p^(2 - alpha).  A group of D / 8 lanes serves a row: each lane holds eight columns of dO_i, fetches its
 // 16 bytes of v_j and k_j, the group adds up the partial dot products on the DPP network, and since delta_i is only
 // known at the end the lanes keep two sums, A = sum u dP k and B = sum u k: dQ_i = (A - delta_i B) / sqrt(D).  Weights
-// and sums are fp32.  delta_i and 1 / sum_j p_ij go to the arrays the dK/dV kernel reads.
+// and sums are fp32.  delta_i and 1 / sum_j p_ij go to the arrays the dense dK/dV kernel reads.
+//
+// Hand-over to the dK/dV kernel (when the stream has a place of its own): the loop over a row's members leaves dP_ij
+// (fp32) in place of each member's score and the score (half precision) in place of its key; behind the row's last
+// member, delta_i and sum p are known and every member gets its pair of weights (p_ij / sum p, u_ij (dP_ij -
+// delta_i)) in the element type; a last pass writes the pairs into the first words of the stream's entries, which
+// held each entry's place in the lists since the sort.
 //
 // Row blocks whose supports outgrow the stream or the lists are flagged and left to attn_bwd_dq_kernel, launched
 // behind, exactly as in the forward; the kernel is persistent and draws row blocks from the same per-XCD counters.
 #pragma once
 #include "attn_bwd_kernel.h"
 #include "attn_sparse_kernel.h"
+
+// The dK/dV kernel on the streams: waves per SIMD and sets of member rows in flight per wave (a set = four members of each
+// of the keys in progress: 36 registers).  Two waves with three sets measured best on the benchmark shapes; three
+// waves leave room for two sets only and were 5 % slower.
+#ifndef ADSP_DKDV_WAVES
+#define ADSP_DKDV_WAVES 2
+#endif
+#ifndef ADSP_DKDV_QUADS
+#define ADSP_DKDV_QUADS 3
+#endif
+// Profiling builds only (-DADSP_DQ_STOP=1 / -DADSP_DKDV_STOP=1 or 2 in the build's extra flags): the dQ kernel skips
+// its loop over the members; the dK/dV kernel on the streams ends a part behind the copy of its pieces (1) or behind
+// the sort (2), so that the stages can be timed by difference.  Such a build computes no gradients.
+#ifndef ADSP_DQ_STOP
+#define ADSP_DQ_STOP 0
+#endif
+#ifndef ADSP_DKDV_STOP
+#define ADSP_DKDV_STOP 0
+#endif
 
 namespace adsp {
 
@@ -26,7 +51,7 @@ __device__ __forceinline__ void dma4s(const void* gbase, uint32_t off, void* lds
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
                :
                : "v"(off), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(base))
-               : "memory", "m0");
+               : "memory");  // (m0 is a reserved register: the compiler sets it itself before each of its own uses)
 }
 
 // sum over a group of LANES (8 or 16) adjacent lanes, left in every lane of the group
@@ -467,6 +492,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           const uint32_t at = row_start[(ent[j].y >> 20) & 31u] + pos[j];
           lval[at] = __builtin_bit_cast(float, ent[j].x);
           lkey[at] = (uint16_t)(ent[j].y & 0xffffu);
+          // (hand-over: the entry's first word becomes its place in the lists until the weights are known)
+          if (p.stream_dir) reinterpret_cast<uint32_t*>(stream + e)[0] = at;
         }
       }
     }
@@ -479,6 +506,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       constexpr int kGroups = 64 / kLPR;  // rows in progress per wave
       constexpr int kDepth = 4;
       const int grp = lane / kLPR, col = lane % kLPR;
+      const bool hand_over = p.stream_dir != nullptr;  // the stream stays for the dK/dV kernel
       const unsigned char* vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2;
       const unsigned char* krows = kglob;
       const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
@@ -500,7 +528,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
       }
+#if ADSP_DQ_STOP == 1
+      for (int r0 = 0; r0 < 0; r0 += kGroups) {
+#else
       for (int r0 = 0; r0 < 32; r0 += kGroups) {
+#endif
         const int r = (int)row_cnt[r0 + grp];
         const bool row_live = wave_row0 + r < L;
         const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
@@ -538,6 +570,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
             usum += u;
             udp = fmaf(u, dp, udp);
             const float wa = u * dp;
+            // (hand-over: dP takes the place of the member's score, and the score, as a half-precision value, the place of its
+            // key; neither is needed again by this loop.  dP stays in fp32: dP - delta cancels most of it.)
+            if (hand_over && col == 0 && eb + j < e_hi) {
+              lval[eb + j] = dp;
+              lkey[eb + j] = __builtin_bit_cast(uint16_t, (_Float16)val[j]);  // (11 bits: p and u are powers of it)
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const float klo = unpack_lo<T>(kk[j][i]), khi = unpack_hi<T>(kk[j][i]);
@@ -549,6 +587,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           }
         }
         const float delta = usum > 0.f ? udp / usum : 0.f;
+        if (hand_over) {
+          // what the dK/dV kernel needs of a member: p / sum p (weight of dO_i in dV_j) and u (dP - delta) (weight of q_i
+          // in dK_j), as a pair of the element type in place of the member's score
+          const float zinv_r = zsum > 0.f ? 1.f / zsum : 0.f;
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          for (int e = e_lo + col; e < e_hi; e += kLPR) {
+            float pr, u;
+            bwd_prob<AM>((float)__builtin_bit_cast(_Float16, lkey[e]) * qs, p.c0, pr, u);
+            reinterpret_cast<uint32_t*>(lval)[e] = pack2<T>(pr * zinv_r, u * (lval[e] - delta));
+          }
+        }
         if (wave_row0 + r < N) {
           float g[8];
 #pragma unroll
@@ -560,6 +610,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
           const size_t at = (size_t)(b * p.Hq + h) * N + wave_row0 + r;
           p.delta[at] = delta;
           p.zinv[at] = zsum > 0.f ? 1.f / zsum : 0.f;
+        }
+      }
+      if (hand_over) {
+        // every stream entry takes its member's pair of weights from the lists (its first word held the place)
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        constexpr int kPer = (SG::kListCap + 63) / 64;
+        uint32_t at[kPer];  // (all loads under way together: one trip to memory, not one per 64 entries)
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = j * 64 + lane;
+          at[j] = 0u;
+          if (e < stream_n)  // (written by this wave: not from its L1)
+            at[j] = __hip_atomic_load(reinterpret_cast<uint32_t*>(stream + e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = j * 64 + lane;
+          if (e < stream_n) reinterpret_cast<uint32_t*>(stream + e)[0] = reinterpret_cast<const uint32_t*>(lval)[at[j] < (uint32_t)SG::kListCap ? at[j] : 0u];
         }
       }
     }
@@ -1038,13 +1108,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         if (key < N) {
 #pragma unroll
           for (int i = 0; i < 8; ++i) acc_k[i] *= p.sm_scale;
-          // fp32 partial rows of this query head (dkdv_reduce_kernel adds up the heads of a K/V head); a later part of
-          // the walk adds to what the earlier ones stored
-          float* o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
-          float* o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+          // fp32 partial rows of this query head (dkdv_reduce_kernel adds up the heads of a K/V head).  While parts of the
+          // walk are still to come the sums stay in the wave's rows of the workgroup's scratch slot, and the next part
+          // adds to them.
+          float* const sc = p.part_scratch + (((size_t)blockIdx.x * NW + wave) * 32 + r) * (2 * D) + col * 8;
           if (seg > 0) {
-            const f32x4 k0 = *reinterpret_cast<const f32x4*>(o0), k1 = *reinterpret_cast<const f32x4*>(o0 + 4);
-            const f32x4 v0 = *reinterpret_cast<const f32x4*>(o1), v1 = *reinterpret_cast<const f32x4*>(o1 + 4);
+            const f32x4 k0 = *reinterpret_cast<const f32x4*>(sc), k1 = *reinterpret_cast<const f32x4*>(sc + 4);
+            const f32x4 v0 = *reinterpret_cast<const f32x4*>(sc + D), v1 = *reinterpret_cast<const f32x4*>(sc + D + 4);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               acc_k[i] += k0[i];
@@ -1053,10 +1123,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
               acc_v[4 + i] += v1[i];
             }
           }
-          *reinterpret_cast<f32x4*>(o0) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
-          *reinterpret_cast<f32x4*>(o0 + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
-          *reinterpret_cast<f32x4*>(o1) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
-          *reinterpret_cast<f32x4*>(o1 + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+          if (done < nt) {
+            *reinterpret_cast<f32x4*>(sc) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
+            *reinterpret_cast<f32x4*>(sc + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
+            *reinterpret_cast<f32x4*>(sc + D) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
+            *reinterpret_cast<f32x4*>(sc + D + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+          } else {
+            float* const o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
+            float* const o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+            __builtin_nontemporal_store(f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]}, reinterpret_cast<f32x4*>(o0));
+            __builtin_nontemporal_store(f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]}, reinterpret_cast<f32x4*>(o0 + 4));
+            __builtin_nontemporal_store(f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]}, reinterpret_cast<f32x4*>(o1));
+            __builtin_nontemporal_store(f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]}, reinterpret_cast<f32x4*>(o1 + 4));
+          }
         }
       }
     }
@@ -1081,21 +1160,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 
 
 
-// dK and dV from the supports the dQ kernel found (16-bit inputs, alpha = 1.5 / 2, head dims 64 / 128): the same work as
-// attn_bwd_dkdv_sparse_kernel without its score walk.  The dQ kernel leaves the stream of every (row block, wave) in
-// place -- (score - threshold, key | row) pairs sorted by 16-key half block -- with a table of where each 32-key block
+// dK and dV from the supports the dQ kernel found (16-bit inputs, alpha = 1.5 / 2, head dims 64 / 128): the same sums as
+// attn_bwd_dkdv_sparse_kernel without its score walk and without its arithmetic per member.  The dQ kernel leaves the
+// stream of every (row block, wave) in place -- per member the pair of weights (p_ij / sum_j p_ij, u_ij (dP_ij -
+// delta_i)) in the element type and key | row, sorted by 16-key half block -- with a table of where each 32-key block
 // starts.  A workgroup serves one (key block, query head); each of its waves owns 32 keys, copies the pieces of all
 // streams of the head that hold its keys (row blocks from its own on with a causal mask) into a stream of its own, as
-// (score - threshold, query | key << 20) pairs, and from there on does what the walking kernel does: a counting sort by
-// key into lists in LDS, and per key the sums over its queries.  A wave that has more members than its lists hold works
-// them off in parts; the waves of a workgroup share nothing and do not wait for each other.  The sums are fp32 partial
-// rows per query head for dkdv_reduce_kernel; where a K/V head has a single query head the last part writes dK and dV
-// in the element type and there is no reduction.  A key block one of whose
-// row blocks the dQ kernel gave up (no stream) is flagged for attn_bwd_dkdv_kernel with all its heads.
-// (three waves per SIMD: the two sets of member rows in flight want 168 registers; with four waves and one set the
-// kernel was 2 % slower, with four waves and two sets it spilled)
+// (weights, query | key << 20) pairs, sorts them by key into lists in LDS (a counting sort) and adds up, per key,
+// weight times dO_i into dV_j and weight times q_i into dK_j: two-term dot products with the weight in one half of the
+// pair, as the dense kernel's matrix products take the weights in the element type.  A wave that has more members than
+// its lists hold works them off in parts (the sums wait in fp32 in the workgroup's scratch slot); the waves of a
+// workgroup share nothing and do not wait for each other.  The sums are fp32 partial rows per query head for
+// dkdv_reduce_kernel; where a K/V head has a single query head the last part writes dK and dV in the element type and
+// there is no reduction.  A key block one of whose row blocks the dQ kernel gave up (no stream) is flagged for
+// attn_bwd_dkdv_kernel with all its heads.
 template <typename T, int D, int AM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_bwd_dkdv_stream_kernel(AttnBwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_WAVES, ADSP_DKDV_WAVES))) void attn_bwd_dkdv_stream_kernel(AttnBwdParams p) {
+  constexpr int kQuads = ADSP_DKDV_QUADS;
   using G = TileGeo<T, D>;
   using SG = SparseGeo<T, D>;
   static_assert(G::k16, "16-bit element types only");
@@ -1274,6 +1355,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
+#if ADSP_DKDV_STOP == 1
+      if (cursor >= n_pairs) break;
+      continue;
+#endif
 
       // ---- the wave's stream -> per-key lists in its share of LDS (a counting sort by key) ---------------------------
       if (lane < 32) row_cnt[lane] = 0u;
@@ -1311,6 +1396,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
+#if ADSP_DKDV_STOP == 2
+      if (cursor >= n_pairs) break;
+      continue;
+#endif
       // The keys are served four at a time (a group of lanes each) and a round lasts as long as its longest list: keys
       // in the order of their list lengths, longest first, keep the four of a round alike.  row_cnt becomes that order.
       {
@@ -1326,108 +1415,88 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         __builtin_amdgcn_wave_barrier();
       }
 
-      // ---- per key: its list holds the queries (of this head) in whose support it lies, with score minus threshold.
-      // A group of D / 8 lanes per key, each lane 8 columns of v_j; per member it fetches its 16 bytes of dO_i and q_i and
-      // the row's delta_i and 1 / sum p (written by the dQ kernels), forms dP_ij = dO_i . v_j across the group and adds
-      // p_ij / sum p * dO_i to dV_j and u_ij (dP_ij - delta_i) * q_i to dK_j. -------------------------------------------
+      // ---- per key: its list holds the queries (of this head) in whose support it lies, each with the pair of weights
+      // the dQ kernel left.  A group of D / 8 lanes per key, each lane 8 columns; per member it fetches its 16 bytes of
+      // dO_i and q_i and adds p_ij / sum p * dO_i to dV_j and u_ij (dP_ij - delta_i) * q_i to dK_j. ----------------------
       {
         constexpr int kLPR = D / 8;         // lanes per key
         constexpr int kGroups = 64 / kLPR;  // keys in progress per wave
         constexpr int kDepth = 4;
         const int grp = lane / kLPR, col = lane % kLPR;
-        const unsigned char* const vrows = reinterpret_cast<const unsigned char*>(p.v) + kv_base * 2;
         const unsigned char* const qrows = reinterpret_cast<const unsigned char*>(p.q) + qo_base * 2;
         const unsigned char* const dorows = reinterpret_cast<const unsigned char*>(p.dout) + qo_base * 2;
-        const unsigned char* const delta_rows = reinterpret_cast<const unsigned char*>(p.delta + (size_t)(b * p.Hq + h) * N);
-        const unsigned char* const zinv_rows = reinterpret_cast<const unsigned char*>(p.zinv + (size_t)(b * p.Hq + h) * N);
         const uint32_t col16 = (uint32_t)col * 16u;  // (32-bit offsets per lane: a head's rows span N * D * 2 <= 16 MB)
-        for (int r0 = 0; r0 < 32; r0 += kGroups) {
-          const int r = (int)row_cnt[r0 + grp];
+        constexpr int kRounds = 32 / kGroups;
+        // The rounds (kGroups keys each, in the order of their list lengths) run as one sequence of member sets: the
+        // fetches stay kQuads - 1 sets ahead across the rounds' borders, so the loads drain once per part and not once
+        // per round.  A round lasts as long as its longest list, the one of its first key; a round without members still
+        // takes one (empty) set, behind which its zero sums are stored.
+        int nq_mine = 1;  // lane i < kRounds: sets of round i
+        if (lane < kRounds) {
+          const int r = (int)row_cnt[lane * kGroups];
+          const int len = (int)(row_start[r + 1] - row_start[r]);
+          nq_mine = len > 0 ? (len + kDepth - 1) / kDepth : 1;
+        }
+        int total = 0;
+#pragma unroll
+        for (int i = 0; i < kRounds; ++i) total += __builtin_amdgcn_readlane(nq_mine, i);
+        float acc_v[8], acc_k[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          acc_v[i] = 0.f;
+          acc_k[i] = 0.f;
+        }
+        struct Quad {
+          u32x4 dd[kDepth], qq[kDepth];
+          uint32_t w[kDepth];  // (p / sum p, u (dP - delta)) in the element type, from the dQ kernel
+        };
+        // the fetching side: round rf, set qf of nqf, the lane's list bounds and a valid query for slots without a member
+        int rf = 0, qf = 0, nqf = __builtin_amdgcn_readlane(nq_mine, 0), fetched = 0;
+        int e_f = 0, e_hi_f = 0;
+        uint32_t safe_q = 0u;
+        auto open_round = [&](int rr) {
+          const int r = (int)row_cnt[rr * kGroups + grp];
           const int key = wave_row0 + r;
-          const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
-          u32x4 vj = {0u, 0u, 0u, 0u};  // the lane's eight columns of v_j
-          if (key < L) vj = *reinterpret_cast<const u32x4*>(vrows + ((uint32_t)key * (uint32_t)(D * 2) + col16));
-          // a slot without a member takes the rows of a valid query with a zero score: no weight, and no branch
-          const uint32_t safe_q = (uint32_t)(key < L ? key : L - 1);
-          float acc_v[8], acc_k[8];
+          e_f = (int)row_start[r];
+          e_hi_f = (int)row_start[r + 1];
+          safe_q = (uint32_t)(key < L ? key : L - 1);
+        };
+        open_round(0);
+        auto fetch_next = [&](Quad& m) {
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            acc_v[i] = 0.f;
-            acc_k[i] = 0.f;
+          for (int j = 0; j < kDepth; ++j) {
+            const bool has = e_f + j < e_hi_f;
+            const uint32_t qidx = has ? (uint32_t)lkey[e_f + j] : safe_q;  // (the list arrays end well inside the wave's LDS)
+            m.w[j] = has ? reinterpret_cast<const uint32_t*>(lval)[e_f + j] : 0u;  // (no member: zero weights, no branch)
+            const uint32_t roff = qidx * (uint32_t)(D * 2) + col16;
+            m.dd[j] = *reinterpret_cast<const u32x4*>(dorows + roff);
+            m.qq[j] = *reinterpret_cast<const u32x4*>(qrows + roff);
           }
-          // Two sets of registers: the rows of the next four members are under way while the sums of the current four are
-          // formed (a wave that waited for its loads before every round left the vector pipe idle a quarter of the time).
-          struct Quad {
-            u32x4 dd[kDepth], qq[kDepth];
-            float val[kDepth], dl[kDepth], zi[kDepth];
-          };
-          auto fetch = [&](Quad& m, int eb) {
-#pragma unroll
-            for (int j = 0; j < kDepth; ++j) {
-              const bool has = eb + j < e_hi;
-              const uint32_t qidx = has ? (uint32_t)lkey[eb + j] : safe_q;  // (the list arrays end well inside the wave's LDS)
-              m.val[j] = has ? lval[eb + j] : 0.f;
-              const uint32_t roff = qidx * (uint32_t)(D * 2) + col16;
-              m.dd[j] = *reinterpret_cast<const u32x4*>(dorows + roff);
-              m.qq[j] = *reinterpret_cast<const u32x4*>(qrows + roff);
-              m.dl[j] = *reinterpret_cast<const float*>(delta_rows + qidx * 4u);
-              m.zi[j] = *reinterpret_cast<const float*>(zinv_rows + qidx * 4u);
-            }
-          };
-          auto consume = [&](const Quad& m) {
-            static_assert(kDepth == 4, "dot8x4 takes four members");
-            float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
-            dot8x4<T>(part, vj, m.dd);
-#pragma unroll
-            for (int j = 0; j < kDepth; ++j) {
-              float dof[8];
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                dof[2 * i] = unpack_lo<T>(m.dd[j][i]);
-                dof[2 * i + 1] = unpack_hi<T>(m.dd[j][i]);
-              }
-              const float dp = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
-              float pr, u;
-              bwd_prob<AM>(m.val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
-              const float ph = pr * m.zi[j], dx = u * (dp - m.dl[j]);
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                acc_v[2 * i] = fmaf(ph, dof[2 * i], acc_v[2 * i]);
-                acc_v[2 * i + 1] = fmaf(ph, dof[2 * i + 1], acc_v[2 * i + 1]);
-                acc_k[2 * i] = fmaf(dx, unpack_lo<T>(m.qq[j][i]), acc_k[2 * i]);
-                acc_k[2 * i + 1] = fmaf(dx, unpack_hi<T>(m.qq[j][i]), acc_k[2 * i + 1]);
-              }
-            }
-          };
-          {
-            Quad m0, m1;
-            int eb = e_lo;
-            if (__builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull) {
-              fetch(m0, eb);
-              for (;;) {
-                eb += kDepth;
-                const bool more1 = __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull;
-                if (more1) fetch(m1, eb);
-                consume(m0);
-                if (!more1) break;
-                eb += kDepth;
-                const bool more0 = __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull;
-                if (more0) fetch(m0, eb);
-                consume(m1);
-                if (!more0) break;
-              }
+          e_f += kDepth;
+          ++fetched;
+          if (++qf == nqf) {
+            qf = 0;
+            ++rf;
+            if (rf < kRounds) {
+              nqf = __builtin_amdgcn_readlane(nq_mine, rf);
+              open_round(rf);
             }
           }
+        };
+        // the consuming side: round rc, set qc of nqc
+        int rc = 0, qc = 0, nqc = __builtin_amdgcn_readlane(nq_mine, 0), consumed = 0;
+        auto store_round = [&](int rr) {
+          const int key = wave_row0 + (int)row_cnt[rr * kGroups + grp];
           if (key < N) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc_k[i] *= p.sm_scale;
-            // fp32 partial rows of this query head (dkdv_reduce_kernel adds up the heads of a K/V head); a later part
-            // adds to what the earlier ones stored
-            float* o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
-            float* o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+            // While parts are still to come the sums stay in fp32, in the wave's rows of the workgroup's scratch slot, and
+            // the next part adds to them.  The last part writes an fp32 partial row of this query head (dkdv_reduce_kernel
+            // adds up the heads of a K/V head), or dK and dV themselves where the head is the only one.
+            float* const sc = p.part_scratch + (((size_t)blockIdx.x * NW + wave) * 32 + (key - wave_row0)) * (2 * D) + col * 8;
             if (seg > 0) {
-              const f32x4 k0 = *reinterpret_cast<const f32x4*>(o0), k1 = *reinterpret_cast<const f32x4*>(o0 + 4);
-              const f32x4 v0 = *reinterpret_cast<const f32x4*>(o1), v1 = *reinterpret_cast<const f32x4*>(o1 + 4);
+              const f32x4 k0 = *reinterpret_cast<const f32x4*>(sc), k1 = *reinterpret_cast<const f32x4*>(sc + 4);
+              const f32x4 v0 = *reinterpret_cast<const f32x4*>(sc + D), v1 = *reinterpret_cast<const f32x4*>(sc + D + 4);
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 acc_k[i] += k0[i];
@@ -1436,16 +1505,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 acc_v[4 + i] += v1[i];
               }
             }
-            if (direct && cursor >= n_pairs) {  // the last part of the only head: the sums in the element type
+            if (cursor < n_pairs) {
+              *reinterpret_cast<f32x4*>(sc) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
+              *reinterpret_cast<f32x4*>(sc + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
+              *reinterpret_cast<f32x4*>(sc + D) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
+              *reinterpret_cast<f32x4*>(sc + D + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+            } else if (direct) {
               const u32x4 wk = {pack2<T>(acc_k[0], acc_k[1]), pack2<T>(acc_k[2], acc_k[3]), pack2<T>(acc_k[4], acc_k[5]), pack2<T>(acc_k[6], acc_k[7])};
               const u32x4 wv = {pack2<T>(acc_v[0], acc_v[1]), pack2<T>(acc_v[2], acc_v[3]), pack2<T>(acc_v[4], acc_v[5]), pack2<T>(acc_v[6], acc_v[7])};
               *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dk) + kv_base + (size_t)key * D + col * 8) = wk;
               *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dv) + kv_base + (size_t)key * D + col * 8) = wv;
             } else {
-              *reinterpret_cast<f32x4*>(o0) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
-              *reinterpret_cast<f32x4*>(o0 + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
-              *reinterpret_cast<f32x4*>(o1) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
-              *reinterpret_cast<f32x4*>(o1 + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
+              // (streamed past the caches: the rows of q and dO that the other key blocks of the head gather stay in L2)
+              float* const o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
+              float* const o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+              __builtin_nontemporal_store(f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]}, reinterpret_cast<f32x4*>(o0));
+              __builtin_nontemporal_store(f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]}, reinterpret_cast<f32x4*>(o0 + 4));
+              __builtin_nontemporal_store(f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]}, reinterpret_cast<f32x4*>(o1));
+              __builtin_nontemporal_store(f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]}, reinterpret_cast<f32x4*>(o1 + 4));
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            acc_v[i] = 0.f;
+            acc_k[i] = 0.f;
+          }
+        };
+        // dV_j += p_ij / sum p * dO_i and dK_j += u_ij (dP_ij - delta_i) * q_i as two-term dot products with the weight
+        // in one half of the pair
+        auto consume_next = [&](const Quad& m) {
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) {
+            dot2_chunk<T>(acc_v, m.dd[j], m.w[j] & 0xffffu, m.w[j] << 16);
+            dot2_chunk<T>(acc_k, m.qq[j], m.w[j] >> 16, m.w[j] & 0xffff0000u);
+          }
+          ++consumed;
+          if (++qc == nqc) {
+            store_round(rc);
+            qc = 0;
+            ++rc;
+            if (rc < kRounds) nqc = __builtin_amdgcn_readlane(nq_mine, rc);
+          }
+        };
+        {
+          Quad ring_q[kQuads];
+#pragma unroll
+          for (int k = 0; k < kQuads - 1; ++k)
+            if (fetched < total) fetch_next(ring_q[k]);
+          while (consumed < total) {
+#pragma unroll
+            for (int k = 0; k < kQuads; ++k) {
+              if (consumed < total) {
+                if (fetched < total) fetch_next(ring_q[(k + kQuads - 1) % kQuads]);
+                consume_next(ring_q[k]);
+              }
             }
           }
         }

@@ -101,7 +101,7 @@ __device__ __forceinline__ void dma16(const void* gsrc, void* lds) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane(base))
-               : "memory", "m0");
+               : "memory");  // (m0 is a reserved register: the compiler sets it itself before each of its own uses)
 }
 
 // The same with the global address split into a wave-uniform base (a scalar register pair) and a 32-bit byte offset per
@@ -119,7 +119,7 @@ __device__ __forceinline__ void dma16s(const void* gbase, uint32_t off, void* ld
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(off), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(base))
-               : "memory", "m0");
+               : "memory");  // (m0 is a reserved register: the compiler sets it itself before each of its own uses)
 }
 
 // 16-byte LDS read at a byte address held as an integer (plus a constant that lands in the instruction's offset field)

@@ -206,7 +206,8 @@ def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B
         else:
             os.environ["ADSP_BWD_STREAMS"] = old
     for a, b in zip(got["1"], got["0"]):
-        assert max_err(a, b.float().cpu(), report=False) < 1.6e-2  # (a unit in the last place of a bf16 value in [1, 2) is 7.8e-3)
+        # (the kernel on the streams takes each member's two weights in the element type, the walking one in fp32)
+        assert max_err(a, b.float().cpu(), report=False) < grad_tol(dtype)
 
 
 @pytest.mark.parametrize("alpha,causal,B,Hq,Hkv,N,D,dtype,lens,version,scale,sparse", [
@@ -241,7 +242,8 @@ def test_backward_with_and_without_the_supports_the_forward_kept(alpha, causal, 
         else:
             os.environ["ADSP_SPARSE"] = old
     for a, b in zip(got["always"], got["never"]):
-        assert max_err(a, b.float().cpu(), report=False) < 1.6e-2  # (a unit in the last place of a bf16 value in [1, 2) is 7.8e-3)
+        # (the kernel on the streams takes each member's two weights in the element type, the walking one in fp32)
+        assert max_err(a, b.float().cpu(), report=False) < grad_tol(dtype)
 
 
 def _both_routes(q, k, v, do, fn):
