@@ -32,9 +32,10 @@
 #ifndef ADSP_DKDV_QUADS
 #define ADSP_DKDV_QUADS 3
 #endif
-// Profiling builds only (-DADSP_DQ_STOP=1 / -DADSP_DKDV_STOP=1 or 2 in the build's extra flags): the dQ kernel skips
-// its loop over the members; the dK/dV kernel on the streams ends a part behind the copy of its pieces (1) or behind
-// the sort (2), so that the stages can be timed by difference.  Such a build computes no gradients.
+// Profiling builds only (-DADSP_DQ_STOP=1 or 2 / -DADSP_DKDV_STOP=1 or 2 in the build's extra flags): the dQ kernel skips
+// its loop over the members (1) or ends a row block in front of the sort (2); the dK/dV kernel on the streams ends a
+// part behind the table of its pieces (1) or behind the sort (2), so that the stages can be timed by difference.  Such
+// a build computes no gradients.
 #ifndef ADSP_DQ_STOP
 #define ADSP_DQ_STOP 0
 #endif
@@ -392,18 +393,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       const int n_fwd = (int)p.fwd_lens[stream_id] < SG::kListCap ? (int)p.fwd_lens[stream_id] : SG::kListCap;
       const uint2* const src = reinterpret_cast<const uint2*>(p.fwd_streams) + stream_id * (size_t)kSparseStreamCap;
       const float t_mine = live ? p.fwd_tshift[(size_t)(b * p.Hq + h) * N + qi] : INFINITY;  // lanes r and r + 32: row r
-      for (int e0 = 0; e0 < n_fwd; e0 += 64) {
-        const int e = e0 + lane;
-        uint2 ent = {0u, 0u};
-        if (e < n_fwd) ent = src[e];
-        const float x = __builtin_bit_cast(float, ent.x) - __shfl(t_mine, (int)((ent.y >> 20) & 31u), 64);
-        const bool keep = e < n_fwd && x > 0.f;
-        const unsigned long long m = __builtin_amdgcn_ballot_w64(keep);
-        if (keep) {
-          const int at = stream_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-          stream[at] = uint2{__builtin_bit_cast(uint32_t, x), ent.y};
+      constexpr int kPerF = (SG::kListCap + 63) / 64;
+      uint2 fe[kPerF];  // (all loads under way together: one trip to memory, not one per 64 entries)
+#pragma unroll
+      for (int j = 0; j < kPerF; ++j) {
+        const int e = j * 64 + lane;
+        fe[j] = uint2{0u, 0u};
+        if (e < n_fwd) fe[j] = src[e];
+      }
+#pragma unroll
+      for (int j = 0; j < kPerF; ++j) {
+        if (j * 64 < n_fwd) {
+          const int e = j * 64 + lane;
+          const uint2 ent = fe[j];
+          const float x = __builtin_bit_cast(float, ent.x) - __shfl(t_mine, (int)((ent.y >> 20) & 31u), 64);
+          const bool keep = e < n_fwd && x > 0.f;
+          const unsigned long long m = __builtin_amdgcn_ballot_w64(keep);
+          if (keep) {
+            const int at = stream_n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+            stream[at] = uint2{__builtin_bit_cast(uint32_t, x), ent.y};
+          }
+          stream_n += __builtin_popcountll(m);
         }
-        stream_n += __builtin_popcountll(m);
       }
     } else {
     walk(std::integral_constant<int, SG::kStages>{}, std::integral_constant<int, G::kKTile>{}, std::integral_constant<int, kKPer>{}, issue_k, [&](int kt, const unsigned char* kt_lds) {
@@ -433,6 +444,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       }
       continue;
     }
+#if ADSP_DQ_STOP == 2
+    continue;
+#endif
 
     // ---- the wave's stream -> per-row lists in its share of LDS (a counting sort by row) ----------------------------
     unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
@@ -1164,9 +1178,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 // attn_bwd_dkdv_sparse_kernel without its score walk and without its arithmetic per member.  The dQ kernel leaves the
 // stream of every (row block, wave) in place -- per member the pair of weights (p_ij / sum_j p_ij, u_ij (dP_ij -
 // delta_i)) in the element type and key | row, sorted by 16-key half block -- with a table of where each 32-key block
-// starts.  A workgroup serves one (key block, query head); each of its waves owns 32 keys, copies the pieces of all
-// streams of the head that hold its keys (row blocks from its own on with a causal mask) into a stream of its own, as
-// (weights, query | key << 20) pairs, sorts them by key into lists in LDS (a counting sort) and adds up, per key,
+// starts.  A workgroup serves one (key block, query head); each of its waves owns 32 keys, looks up the pieces of all
+// streams of the head that hold its keys (row blocks from its own on with a causal mask), fetches their entries -- all
+// loads under way together, an entry finds its piece by a binary search in a table of the pieces in LDS -- sorts them
+// by key into lists in LDS (a counting sort of (weights, query) pairs) and adds up, per key,
 // weight times dO_i into dV_j and weight times q_i into dK_j: two-term dot products with the weight in one half of the
 // pair, as the dense kernel's matrix products take the weights in the element type.  A wave that has more members than
 // its lists hold works them off in parts (the sums wait in fp32 in the workgroup's scratch slot); the waves of a
@@ -1285,74 +1300,55 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
     const size_t head_stream0 = (size_t)(b * p.Hq + h) * n_mblk * NW;  // first stream of the head
     const uint2* const src_streams = reinterpret_cast<const uint2*>(p.streams) + head_stream0 * (size_t)kSparseStreamCap;
     const uint16_t* const src_dir = p.stream_dir + head_stream0 * (size_t)p.dir_stride + k32;
-    uint2* const stream = reinterpret_cast<uint2*>(p.events) + ((size_t)blockIdx.x * NW + wave) * (size_t)kSparseStreamCap;
 
     unsigned char* const wave_lds = lds_all + wave * SG::kWaveLds;
-    float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap scores minus the threshold
+    float* const lval = reinterpret_cast<float*>(wave_lds);                                  // kListCap pairs of weights
     uint16_t* const lkey = reinterpret_cast<uint16_t*>(wave_lds + SG::kListCap * 4);         // their queries
     uint32_t* const row_cnt = reinterpret_cast<uint32_t*>(wave_lds + SG::kListCap * 6);     // 32 counters
     uint32_t* const row_start = row_cnt + 32;                                                // 33 offsets
-    // while the pieces are copied the lists' room holds, per piece of the batch: entries up to and including it, where
-    // it starts among the head's streams, and the first query row of its stream
-    uint32_t* const pc_incl = reinterpret_cast<uint32_t*>(wave_lds);
-    uint32_t* const pc_src = pc_incl + 64;
-    uint32_t* const pc_row = pc_src + 64;
-    static_assert(SG::kListCap * 4 >= 3 * 64 * 4, "room for the batch table");
+    // while a part's entries are fetched the lists' room holds a table of its pieces: entries up to and including the
+    // piece, and where the piece starts in its stream (which stream, and its first query row, follow from the piece's
+    // number)
+    constexpr int kTab = 1024;
+    uint16_t* const pc_incl = reinterpret_cast<uint16_t*>(wave_lds);
+    uint16_t* const pc_lo = pc_incl + kTab;
+    static_assert(SG::kListCap * 4 >= 2 * kTab * 2 && SG::kListCap < 65536, "room for the table of pieces, 16-bit counts");
 
     int cursor = 0;  // next piece (wave-uniform)
     for (int seg = 0;; ++seg) {
-      int stream_n = 0;  // wave-uniform
-      while (cursor < n_pairs) {
+      // ---- the pieces of this part: as many as the lists and the table hold ----------------------------------------
+      int stream_n = 0, n_tab = 0;  // wave-uniform
+      const int cursor0 = cursor;   // first piece of the part
+      while (cursor < n_pairs && n_tab < kTab) {
         const int pi = cursor + lane;
-        uint32_t len = 0u, src = 0u, row0 = 0u;
+        uint32_t len = 0u, lo = 0u;
         if (pi < n_pairs) {
           // from the last row block down: a key block holds about as many members in a row block as any other key block
           // of its head does, so the key blocks of a head that run side by side ask for the same rows of q and dO at
           // about the same time, whichever key block they are (a tenth fewer L2 misses than from the first one up)
           const int rb = rb_hi - pi / NW, w = pi % NW;
           const size_t sid = (size_t)rb * NW + w;
-          uint32_t lo = src_dir[sid * (size_t)p.dir_stride], hi = src_dir[sid * (size_t)p.dir_stride + 1];
+          uint32_t hi = src_dir[sid * (size_t)p.dir_stride + 1];
+          lo = src_dir[sid * (size_t)p.dir_stride];
           hi = hi < (uint32_t)SG::kListCap ? hi : (uint32_t)SG::kListCap;  // (what the dQ kernel wrote lies within these bounds)
           lo = lo < hi ? lo : hi;
           len = hi - lo;
-          src = (uint32_t)(sid * (size_t)kSparseStreamCap) + lo;
-          row0 = (uint32_t)(rb * BM + w * 32);
         }
         const int incl = wave_scan_i((int)len);
         // the pieces of this batch that still fit (the sums grow with the lane: a run of lanes from 0 on)
-        const unsigned long long fm = __builtin_amdgcn_ballot_w64(pi < n_pairs && stream_n + incl <= SG::kListCap);
+        const unsigned long long fm = __builtin_amdgcn_ballot_w64(pi < n_pairs && n_tab + lane < kTab && stream_n + incl <= SG::kListCap);
         const int m = __builtin_popcountll(fm);
-        if (m == 0) break;  // (the stream is not empty then: a single piece is no longer than a list)
+        if (m == 0) break;  // (the part is not empty then: a single piece is no longer than a list)
         const int batch = __builtin_amdgcn_readlane(incl, m - 1);
-        __builtin_amdgcn_wave_barrier();
         if (lane < m) {
-          pc_incl[lane] = (uint32_t)incl;
-          pc_src[lane] = src;
-          pc_row[lane] = row0;
+          pc_incl[n_tab + lane] = (uint16_t)(stream_n + incl);
+          pc_lo[n_tab + lane] = (uint16_t)lo;
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int e0 = 0; e0 < batch; e0 += 64) {
-          const int e = e0 + lane;
-          if (e < batch) {
-            int a = 0, z = m - 1;  // the piece that holds entry e: the first one whose running sum exceeds e
-            while (a < z) {
-              const int mid = (a + z) >> 1;
-              if (pc_incl[mid] > (uint32_t)e) z = mid;
-              else a = mid + 1;
-            }
-            const uint32_t before = a ? pc_incl[a - 1] : 0u;
-            const uint2 ent = src_streams[pc_src[a] + ((uint32_t)e - before)];
-            const uint32_t key = ent.y & 0xffffu, row = (ent.y >> 20) & 31u;
-            stream[stream_n + e] = uint2{ent.x, (pc_row[a] + row) | ((key - (uint32_t)wave_row0) << 20)};
-          }
-        }
-        __builtin_amdgcn_wave_barrier();
         stream_n += batch;
+        n_tab += m;
         cursor += m;
         if (m < 64) break;  // the next piece does not fit, or there is none
       }
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // the wave's stream is in memory before it reads it back
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
 #if ADSP_DKDV_STOP == 1
@@ -1360,17 +1356,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
       continue;
 #endif
 
-      // ---- the wave's stream -> per-key lists in its share of LDS (a counting sort by key) ---------------------------
+      // ---- the part's entries, all fetches under way together, -> per-key lists in the wave's share of LDS (a counting
+      // sort by key).  Entry e of the part lies in the first piece whose running sum exceeds e. ------------------------
       if (lane < 32) row_cnt[lane] = 0u;
       {
         constexpr int kPer = (SG::kListCap + 63) / 64;
         uint2 ent[kPer];
+        uint32_t rowv[kPer];
         uint32_t pos[kPer];
 #pragma unroll
         for (int j = 0; j < kPer; ++j) {
           const int e = j * 64 + lane;
           ent[j] = uint2{0u, 0u};
-          if (e < stream_n) ent[j] = stream[e];
+          rowv[j] = 0u;
+          if (e < stream_n) {
+            int a = 0;  // pieces whose running sum is <= e
+#pragma unroll
+            for (int step = kTab / 2; step >= 1; step >>= 1) {
+              const int t = a + step;
+              if (t <= n_tab && (int)pc_incl[t - 1] <= e) a = t;
+            }
+            const int before = a ? (int)pc_incl[a - 1] : 0;
+            const int pi = cursor0 + a, rb = rb_hi - pi / NW, w = pi % NW;
+            ent[j] = src_streams[(uint32_t)(rb * NW + w) * (uint32_t)kSparseStreamCap + (uint32_t)pc_lo[a] + (uint32_t)(e - before)];
+            rowv[j] = (uint32_t)(rb * BM + w * 32);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();  // (the table is read: its room becomes the lists)
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {  // (weights, query | key << 20)
+          const uint32_t key = ent[j].y & 0xffffu, row = (ent[j].y >> 20) & 31u;
+          ent[j].y = (rowv[j] + row) | ((key - (uint32_t)wave_row0) << 20);
         }
 #pragma unroll
         for (int j = 0; j < kPer; ++j) {
@@ -1564,8 +1581,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
         }
       }
       if (cursor >= n_pairs) break;
-      // (the partial rows just written are read back by the next part, by this wave: the wait for its stores at the end
-      // of the next copy comes before those reads)
+      // (the sums just written to the scratch slot are read back by the next part, by this wave: its stores have landed
+      // before the next part begins; every lane is done with the lists)
+      __builtin_amdgcn_s_waitcnt(0x0f70);
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
