@@ -35,10 +35,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these
 # same workloads, each counter scaled by what it reads for a plain 1 GiB copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
-MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.467e9, "c3": 0.5079e9, "c5": 0.577e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5371e9,
+MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.402e9, "c3": 0.5083e9, "c5": 0.559e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5370e9,
                               "c2_bwd_f32": 1.0847e9, "c2_bwd_bf16": 0.5476e9,
-                              "c4_bwd": 15.4e9,
-                              "c5_bwd": 0.962e9}  # c4_bwd: sparse dq kernel 2.33e9 + dk/dv kernel on its streams 11.40e9 + reduction 1.72e9
+                              "c4_bwd": 11.14e9,
+                              "c5_bwd": 0.861e9}  # c4_bwd: sparse dq kernel 3.43e9 + dk/dv kernel on its streams 5.97e9 + reduction 1.74e9
 
 
 # The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a
