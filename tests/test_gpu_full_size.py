@@ -169,3 +169,32 @@ def test_fp32_long_context_forward_and_backward(seq_len):
     assert (qg.grad[0, 0][rest.to(DEV)] == 0).all()  # rows without an upstream gradient
     assert (kg.grad[0, 0].double().cpu() - dx.t() @ qd * sm).abs().max().item() < 1e-4
     assert (vg.grad[0, 0].double().cpu() - probs.t() @ dod).abs().max().item() < 1e-4
+
+
+def test_bf16_longest_context_backward_on_the_supports():
+    """N = 65536, the longest sequence the sparse-support kernels take (16-bit key indices; the dK/dV kernel's table of
+    pieces is filled more than once per key block here), D = 64, bf16, causal: forward and backward with an upstream
+    gradient that is non-zero on 96 sampled rows only, so that dq on those rows and dk, dv everywhere follow from the
+    sampled rows' probabilities alone (as in the fp32 long-context test above).  2e-2 / 4e-2 on the magnitude-aware scale."""
+    g = torch.Generator().manual_seed(5)
+    N, D = 65536, 64
+    q, k, v = (torch.randn(1, 1, N, D, generator=g).to(torch.bfloat16) for _ in range(3))
+    rows = sorted(set([0, 1, 127, 128, N // 2, N - 129, N - 2, N - 1] + torch.randint(0, N, (88,), generator=g).tolist()))
+    do = torch.zeros(1, 1, N, D, dtype=torch.bfloat16)
+    do[0, 0, rows] = torch.randn(len(rows), D, generator=g).to(torch.bfloat16)
+    qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    out = A.adasplash_v2(qg, kg, vg, niter=1)
+    out.backward(do.to(DEV))
+    z, tau, probs = _oracle_rows(q, k, 0, 0, rows, 1.5, True, N)
+    kd, vd, dod, qd = k[0, 0].double(), v[0, 0].double(), do[0, 0, rows].double(), q[0, 0, rows].double()
+    assert max_err(out[0, 0, rows].detach(), probs @ vd) < 2e-2
+    u = probs.sqrt()
+    dp = dod @ vd.t()
+    dx = u * (dp - (u * dp).sum(-1, keepdim=True) / u.sum(-1, keepdim=True))
+    sm = 1.0 / math.sqrt(D)
+    assert max_err(qg.grad[0, 0, rows], dx @ kd * sm) < 4e-2
+    rest = torch.ones(N, dtype=torch.bool)
+    rest[rows] = False
+    assert (qg.grad[0, 0][rest.to(DEV)] == 0).all()  # rows without an upstream gradient
+    assert max_err(kg.grad[0, 0], dx.t() @ qd * sm) < 4e-2
+    assert max_err(vg.grad[0, 0], probs.t() @ dod) < 4e-2
