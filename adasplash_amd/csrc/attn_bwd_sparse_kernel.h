@@ -32,10 +32,12 @@
 #ifndef ADSP_DKDV_QUADS
 #define ADSP_DKDV_QUADS 3
 #endif
-// Profiling builds only (-DADSP_DQ_STOP=1 or 2 / -DADSP_DKDV_STOP=1 or 2 in the build's extra flags): the dQ kernel skips
-// its loop over the members (1) or ends a row block in front of the sort (2); the dK/dV kernel on the streams ends a
-// part behind the table of its pieces (1) or behind the sort (2), so that the stages can be timed by difference.  Such
-// a build computes no gradients.
+// Profiling builds only (-DADSP_DQ_STOP=1 .. 3 / -DADSP_DKDV_STOP=1 .. 3 in the build's extra flags): the dQ kernel skips
+// its loop over the members (1), ends a row block in front of the sort (2) or right behind its set-up (3); the dK/dV
+// kernel on the streams ends a part behind the table of its pieces (1) or behind the sort (2), or an item behind its
+// set-up (3), so that the stages can be timed by difference.  Such a build computes no gradients.  (Items that do
+// nothing are bound by the eight work counters, 2048 increments each at c4's size: the floor of such a build says
+// little about the full kernels.)
 #ifndef ADSP_DQ_STOP
 #define ADSP_DQ_STOP 0
 #endif
@@ -386,6 +388,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         }
       }
     };
+#if ADSP_DQ_STOP == 3
+    continue;
+#endif
     if (from_fwd) {
       // The forward's stream of this row block and wave holds every score above a lower bound of the rows' thresholds,
       // as (score - bound, key | row) pairs in the order of its walk, and the forward left every row's threshold minus
@@ -1294,6 +1299,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
         continue;
       }
     }
+#if ADSP_DKDV_STOP == 3
+    continue;
+#endif
     const int wave_row0 = m0 + wave * 32;
     const int k32 = wave_row0 / 32;
     const int n_pairs = (rb_hi - rb_lo + 1) * NW;  // (row block, wave of the dQ kernel) in order
