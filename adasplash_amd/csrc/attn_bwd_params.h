@@ -35,7 +35,7 @@ struct AttnBwdParams {
   float* part_scratch;  // [slots, waves, 32, 2 D]
   // hand-over of the supports from the dQ kernel to the dK/dV kernel (null: the dK/dV kernel walks for itself): the dQ
   // kernel's streams kept per (row block, wave) instead of per workgroup, and per stream the offsets of the 32-key blocks
-  unsigned char* streams;  // [B, Hq, n_mblk, waves, stream capacity] (score - threshold, key | row << 20) pairs
+  unsigned char* streams;  // [B, Hq, n_mblk, waves, stream capacity] per member (weights, key | row << 20): the pair p / sum p, u (dP - delta) in the element type
   uint16_t* stream_dir;    // [B, Hq, n_mblk, waves, dir_stride]: entry k = first stream entry with key >= 32 k
   int dir_stride;          // 4 n_mblk + 1 offsets, rounded up to an even count
   // supports the forward kept (null: none; see AttnParams): where the flag of a row block is 1 the dQ kernel takes

@@ -184,9 +184,10 @@ int adsp_attn_bwd_kept(const void* q, const void* k, const void* v, const void* 
 /*
  * Workspace of adsp_attn_bwd in bytes; 0 for fp32 and for the head dims the sparse-support kernels do not serve (then
  * `workspace` may be NULL).  For the 16-bit element types at head dims 64 and 128 (sequences of up to 65536 keys): the
- * counters, flags and candidate streams of the sparse-support backward kernels, fp32 partial rows of dk and dv per
- * query head (2 * B * Hq * N * D * 4 bytes), and the supports the dq kernel hands to the dk/dv kernel: per query row
- * block of 128 rows 51 KiB of (score, key) pairs and a table of 4 * ceil(N / 128) + 2 16-bit offsets per wave.
+ * counters, flags and candidate streams of the sparse-support backward kernels, 1024 * D bytes of fp32 sums per
+ * workgroup (items that are worked off in parts), fp32 partial rows of dk and dv per query head (2 * B * Hq * N * D * 4 bytes;
+ * none where Hq == Hkv), and the supports the dq kernel hands to the dk/dv kernel: per query row block of 128 rows
+ * 51 KiB of (weights, key) pairs and a table of 4 * ceil(N / 128) + 2 16-bit offsets per wave.
  * 16-byte aligned device memory; contents need not survive between calls; concurrent calls need a buffer each.
  */
 size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
