@@ -504,8 +504,8 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     w.queue_off = align256(w.copies_bytes);
     w.flags_off = align256(w.queue_off + 256 + ((size_t)B * Hkv + 1) * 8);
     w.events_off = align256(w.flags_off + (size_t)items * 4);
-    // the dK/dV kernel: control words and hint counters of its own, a flag per (K/V head, key block), and fp32
-    // partial rows of dK and dV per query head
+    // the dK/dV kernel: control words and the probe's verdict per K/V head once more, a flag per (K/V head, key
+    // block), fp32 sums per workgroup and fp32 partial rows of dK and dV per query head
     w.queue2_off = align256(w.events_off + (size_t)slots * kSparseSlotBytes);
     w.kvflags_off = align256(w.queue2_off + 256 + ((size_t)B * Hkv + 1) * 8);
     // (fp32 sums of an item worked off in parts: 32 rows of dK | dV per wave of every workgroup)
@@ -522,8 +522,8 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
   return w;
 }
 
-// Clears the control words, hint counters and key-block flags of the sparse-support dK/dV kernel; the K/V heads the
-// probe marked as dense (in the dQ kernel's hint words) stay marked.
+// Clears the control words and key-block flags of the sparse-support dK/dV kernel and copies the probe's verdict per
+// K/V head (the dQ kernel's words) into the kernel's own.
 __global__ __launch_bounds__(256) void bwd_ctrl_clear_kernel(uint32_t* ctrl2, const uint32_t* hints1, int units, int32_t* kv_flags,
                                                             long long n_flags) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;

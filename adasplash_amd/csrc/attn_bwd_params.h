@@ -22,7 +22,7 @@ struct AttnBwdParams {
   // the sparse-support dQ kernel and its hand-over to the dense one (null: dense kernels only), as in AttnParams
   int32_t* block_flags;   // [B, Hq, n_mblk] 1 = row block left to attn_bwd_dq_kernel
   uint32_t* queue;        // control words: work counters, flagged count, "every head dense"
-  uint32_t* hints;        // two counters per K/V head and one pair over all heads
+  uint32_t* hints;        // two words per K/V head: word 0 is 1 << 20 where the probe left the head to the dense kernels
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
   // the sparse-support dK/dV kernel: a control block of its own, one flag per (K/V head, key block), fp32 partial rows
   // [B, Hq, N, D] when a K/V head serves several query heads (null otherwise), and per workgroup and wave 32 fp32

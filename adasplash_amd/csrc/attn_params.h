@@ -39,8 +39,7 @@ struct AttnParams {
   // 1 = left to attn_fwd_kernel, which skips the others when block_flags is set.
   int32_t* block_flags;   // [B, Hq, n_mblk], or null: attn_fwd_kernel serves every row block
   uint32_t* queue;        // eight work counters, one per XCD, then the two control words above; zero at launch
-  uint32_t* hints;        // [B * Hkv + 1][2]: word 0 of a K/V head is 1 << 20 when the probe leaves all of it to the dense kernel (the backward's
-                          // kernels also count row blocks {given up, served} per K/V head and over all heads here); zero at launch
+  uint32_t* hints;        // [B * Hkv + 1][2]: word 0 of a K/V head is 1 << 20 when the probe leaves all of it to the dense kernel, else 0
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
   const unsigned char* k8;  // fp8 (e4m3) copy of K, [B * Hkv][Npad][D] bytes, rows past N zero: the operand of the first walk
   // Four floats per K/V head, set by the probe: powers of two for q and for k (they are multiplied by them before
