@@ -76,6 +76,18 @@ template <> __device__ __forceinline__ void dot8x4<bf16_t>(float (&p)[4], u32x4 
 template <> __device__ __forceinline__ void dot8x4<f16_t>(float (&p)[4], u32x4 a, const u32x4 (&b)[4]) { ADSP_DOT8X4("v_dot2c_f32_f16"); }
 #undef ADSP_DOT8X4
 
+// Sixteen independent 4 x 4 x 4 products on the matrix pipe (a block = four neighbouring lanes): lane 4 b + i holds row i
+// of A_b (four values along k) and column i of B_b; its four result registers are column i of D_b = A_b B_b + C_b.
+typedef short mfma4_s4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4_t mfma4_bf16(u32x2_t a, u32x2_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(mfma4_s4, a), __builtin_bit_cast(mfma4_s4, b), c, 0, 0, 0);
+}
+// x as the sum of two bf16 values (16 bits of x in all): the leading one, or what is left of x behind it
+__device__ __forceinline__ uint32_t bf16_part(float x, bool rest) {
+  const float hi = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & 0xffff0000u);
+  return __builtin_bit_cast(uint32_t, rest ? x - hi : hi) >> 16;
+}
+
 template <int LANES> __device__ __forceinline__ float group_sum(float x) {
   if constexpr (LANES == 16) {
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xf, 0xf, false));  // row_mirror
@@ -557,52 +569,99 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         const int e_lo = (int)row_start[r], e_hi = (int)row_start[r + 1];
         u32x4 dov = {0u, 0u, 0u, 0u};  // the lane's eight columns of dO_i (rows past the valid length may hold anything: not read)
         if (row_live) dov = *reinterpret_cast<const u32x4*>(dorows + (size_t)r * (D * 2));
+        // A = sum u dP k and B = sum u k.  bf16: on the matrix pipe, idle in this kernel -- per column of the lane a
+        // 4 x 4 x 4 product whose k runs over the four members in flight, whose A rows are the weights u dP and u, each
+        // split into two bf16 values (lane 4 b + i of a block supplies row i: the weights lose nothing that a 16-bit
+        // result could show), and whose B column is the members' K values at that column; register i of the result adds
+        // up weight i times K.  f16 (whose exponent range the weights can leave): fp32 multiply-adds.
+        constexpr bool kOnMatrixPipe = std::is_same<T, bf16_t>::value;
         float acc_a[8], acc_b[8];
+        f32x4_t acc4[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           acc_a[i] = 0.f;
           acc_b[i] = 0.f;
+          acc4[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
+        const bool kind_u = (lane & 2) != 0, kind_rest = (lane & 1) != 0;
         float zsum = 0.f, usum = 0.f, udp = 0.f;
-        for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+        // (the rows of a round come longest list first: the first group's row sets the number of turns)
+        const int n_turns = (__builtin_amdgcn_readfirstlane(e_hi - e_lo) + kDepth - 1) / kDepth;
+        for (int turn = 0; turn < n_turns; ++turn) {
+          const int eb = e_lo + turn * kDepth;
+          // (a group whose list has ended reads on without a condition, at a place inside the wave's LDS)
+          const int ebr = eb < SG::kListCap ? eb : SG::kListCap;
           u32x4 vv[kDepth], kk[kDepth];
           float val[kDepth];
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
             // a slot without a member takes the first key's rows (always valid) with a zero score: no weight, no branch
             const bool has = eb + j < e_hi;
-            const uint32_t key = has ? (uint32_t)lkey[eb + j] : 0u;  // (the list arrays end well inside the wave's LDS)
-            val[j] = has ? lval[eb + j] : 0.f;
+            const uint32_t kraw = (uint32_t)lkey[ebr + j];
+            const float vraw = lval[ebr + j];
+            const uint32_t key = has ? kraw : 0u;
+            val[j] = has ? vraw : 0.f;
             const uint32_t roff = key * (uint32_t)(D * 2) + col16;
             vv[j] = *reinterpret_cast<const u32x4*>(vrows + roff);
             kk[j] = *reinterpret_cast<const u32x4*>(krows + roff);
           }
-          static_assert(kDepth == 4, "dot8x4 takes four members");
+          static_assert(kDepth == 4, "dot8x4 and the 4 x 4 x 4 products take four members");
           float part[kDepth] = {0.f, 0.f, 0.f, 0.f};
           dot8x4<T>(part, dov, vv);
+          float dp[kDepth], uu[kDepth];
+#pragma unroll
+          for (int j = 0; j < kDepth; ++j) dp[j] = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
-            const float dp = group_sum<kLPR>(part[j]);  // dO_i . v_j, in every lane of the group
-            float pr, u;
-            bwd_prob<AM>(val[j] * qs, p.c0, pr, u);  // (an absent member has val = 0: p = u = 0)
+            float pr;
+            bwd_prob<AM>(val[j] * qs, p.c0, pr, uu[j]);  // (an absent member has val = 0: p = u = 0)
             zsum += pr;
-            usum += u;
-            udp = fmaf(u, dp, udp);
-            const float wa = u * dp;
-            // (hand-over: dP takes the place of the member's score, and the score, as a half-precision value, the place of its
-            // key; neither is needed again by this loop.  dP stays in fp32: dP - delta cancels most of it.)
-            if (hand_over && col == 0 && eb + j < e_hi) {
-              lval[eb + j] = dp;
-              lkey[eb + j] = __builtin_bit_cast(uint16_t, (_Float16)val[j]);  // (11 bits: p and u are powers of it)
-            }
+            usum += uu[j];
+            udp = fmaf(uu[j], dp[j], udp);
+          }
+          // (hand-over: dP takes the place of the member's score, and the score, as a half-precision value, the place of its
+          // key; neither is needed again by this loop.  dP stays in fp32: dP - delta cancels most of it.)
+          if (hand_over && col == 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float klo = unpack_lo<T>(kk[j][i]), khi = unpack_hi<T>(kk[j][i]);
-              acc_a[2 * i] = fmaf(wa, klo, acc_a[2 * i]);
-              acc_a[2 * i + 1] = fmaf(wa, khi, acc_a[2 * i + 1]);
-              acc_b[2 * i] = fmaf(u, klo, acc_b[2 * i]);
-              acc_b[2 * i + 1] = fmaf(u, khi, acc_b[2 * i + 1]);
+            for (int j = 0; j < kDepth; ++j) {
+              if (eb + j < e_hi) {
+                lval[eb + j] = dp[j];
+                lkey[eb + j] = __builtin_bit_cast(uint16_t, (_Float16)val[j]);  // (11 bits: p and u are powers of it)
+              }
             }
+          }
+          if constexpr (kOnMatrixPipe) {
+            uint32_t w16[kDepth];
+#pragma unroll
+            for (int j = 0; j < kDepth; ++j) w16[j] = bf16_part(kind_u ? uu[j] : uu[j] * dp[j], kind_rest);
+            const u32x2_t aw = {w16[0] | (w16[1] << 16), w16[2] | (w16[3] << 16)};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // (the members' values at an even and at an odd column: the low and the high halves)
+              const u32x2_t b_even = {__builtin_amdgcn_perm(kk[1][i], kk[0][i], 0x05040100u), __builtin_amdgcn_perm(kk[3][i], kk[2][i], 0x05040100u)};
+              const u32x2_t b_odd = {__builtin_amdgcn_perm(kk[1][i], kk[0][i], 0x07060302u), __builtin_amdgcn_perm(kk[3][i], kk[2][i], 0x07060302u)};
+              acc4[2 * i] = mfma4_bf16(aw, b_even, acc4[2 * i]);
+              acc4[2 * i + 1] = mfma4_bf16(aw, b_odd, acc4[2 * i + 1]);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < kDepth; ++j) {
+              const float wa = uu[j] * dp[j];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const float klo = unpack_lo<T>(kk[j][i]), khi = unpack_hi<T>(kk[j][i]);
+                acc_a[2 * i] = fmaf(wa, klo, acc_a[2 * i]);
+                acc_a[2 * i + 1] = fmaf(wa, khi, acc_a[2 * i + 1]);
+                acc_b[2 * i] = fmaf(uu[j], klo, acc_b[2 * i]);
+                acc_b[2 * i + 1] = fmaf(uu[j], khi, acc_b[2 * i + 1]);
+              }
+            }
+          }
+        }
+        if constexpr (kOnMatrixPipe) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            acc_a[i] = acc4[i][0] + acc4[i][1];
+            acc_b[i] = acc4[i][2] + acc4[i][3];
           }
         }
         const float delta = usum > 0.f ? udp / usum : 0.f;

@@ -819,21 +819,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
       const float target = (AM == ATT_15) ? inv_qs * inv_qs : inv_qs;
       // (any alpha: the steps shrink like 1 - 1 / c0 while f is large, so the rounds are more; the launch keeps alphas
       // whose c0 = 1 / (alpha - 1) exceeds 8 on the dense kernel)
+      // (four of the lane's entries per turn, read together; the longest list of the wave sets the number of turns, and
+      // a lane past its list's end reads on inside the wave's LDS and takes -inf)
+      const int max_len = (int)wave_max((float)(row_end - row_lo));
       for (int it = 0; it < (AM == ATT_GEN ? 96 : 24); ++it) {
         float a0 = 0.f, a1 = 0.f;
-        for (int e = row_lo + lh; e < row_end; e += 2) {
-          const float u = fmaxf(lval[e] - t, 0.f);
-          if constexpr (AM == ATT_15) {
-            a0 = fmaf(u, u, a0);
-            a1 += u;
-          } else if constexpr (AM == ATT_2) {
-            a0 += u;
-            a1 += u > 0.f ? 1.f : 0.f;
-          } else {
-            const float uz = u * qs;
-            const float pw = u > 0.f ? fast_exp2(p.c0 * fast_log2(uz)) : 0.f;
-            a0 += pw;
-            a1 += u > 0.f ? pw * fast_rcp(uz) : 0.f;
+        for (int o = 0; o < max_len; o += 8) {
+          const int e0 = row_lo + lh + o;
+          const int e0r = e0 < SG::kListCap ? e0 : SG::kListCap;
+          float x[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float raw = lval[e0r + 2 * j];
+            x[j] = e0 + 2 * j < row_end ? raw : -INFINITY;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float u = fmaxf(x[j] - t, 0.f);
+            if constexpr (AM == ATT_15) {
+              a0 = fmaf(u, u, a0);
+              a1 += u;
+            } else if constexpr (AM == ATT_2) {
+              a0 += u;
+              a1 += u > 0.f ? 1.f : 0.f;
+            } else {
+              const float uz = u * qs;
+              const float pw = u > 0.f ? fast_exp2(p.c0 * fast_log2(uz)) : 0.f;
+              a0 += pw;
+              a1 += u > 0.f ? pw * fast_rcp(uz) : 0.f;
+            }
           }
         }
         a0 += __shfl_xor(a0, 32, 64);
@@ -905,15 +919,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-        for (int eb = e_lo; __builtin_amdgcn_ballot_w64(eb < e_hi) != 0ull; eb += kDepth) {
+        // (the rows of a round come longest support first: the first group's row sets the number of turns)
+        const int n_turns = (__builtin_amdgcn_readfirstlane(e_hi - e_lo) + kDepth - 1) / kDepth;
+        for (int turn = 0; turn < n_turns; ++turn) {
+          const int eb = e_lo + turn * kDepth;
+          // (a group whose list has ended reads on without a condition, at a place inside the wave's LDS)
+          const int ebr = eb < SG::kListCap ? eb : SG::kListCap;
           u32x4 vv[kDepth];
           uint32_t pw[kDepth];
 #pragma unroll
           for (int j = 0; j < kDepth; ++j) {
             // a slot without a member takes the first key's row (always valid) with a zero weight: no zeroing, no branch
             const bool has = eb + j < e_hi;
-            const uint32_t key = has ? (uint32_t)lkey[eb + j] : 0u;  // (the list arrays end well inside the wave's LDS)
-            pw[j] = has ? __builtin_bit_cast(uint32_t, lval[eb + j]) : 0u;
+            const uint32_t kraw = (uint32_t)lkey[ebr + j];
+            const uint32_t wraw = __builtin_bit_cast(uint32_t, lval[ebr + j]);
+            const uint32_t key = has ? kraw : 0u;
+            pw[j] = has ? wraw : 0u;
             vv[j] = *reinterpret_cast<const u32x4*>(vrows + (key * (uint32_t)(D * 2) + col16));
           }
 #pragma unroll
