@@ -127,7 +127,7 @@ def launch_backward(q, k, v, dout, taus, bmask, *, alpha, is_causal, varlen, sup
     dv = torch.empty_like(v)
     delta = torch.empty((B, Hq, N), device=q.device, dtype=torch.float32)
     zinv = torch.empty((B, Hq, N), device=q.device, dtype=torch.float32)
-    ws_bytes = lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dt)
+    ws_bytes = lib.adsp_attn_bwd_workspace_bytes_causal(B, Hq, Hkv, N, D, dt, 1 if is_causal else 0)
     ws = torch.empty((ws_bytes,), device=q.device, dtype=torch.uint8) if ws_bytes else None
     with _lib.device_guard(q.device):
         if supports is not None:

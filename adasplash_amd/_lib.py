@@ -40,6 +40,7 @@ _SIGNATURES = {
     "adsp_attn_bwd_kept": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                                 _dbl, _i, _vp, _sz, _vp, _sz, _vp]),
     "adsp_attn_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "adsp_attn_bwd_workspace_bytes_causal": (_sz, [_i, _i, _i, _i, _i, _i, _i]),
     "adsp_attn_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _dbl,
                            _i, _vp, _sz, _vp]),
 }

@@ -280,6 +280,15 @@ static bool bwd_streams_enabled() {
   return !(e && strcmp(e, "0") == 0);
 }
 
+// With a causal mask the kernel on the dQ kernel's streams serves the key blocks from this share (in 256ths) of a
+// sequence on with one item for all query heads of a K/V head (attn_bwd_dkdv_stream_kernel).  ADSP_DKDV_MERGE256 in the
+// environment overrides it (0: every key block per query head, with partial rows; for comparisons and tests).
+static int dkdv_merge256() {
+  const char* e = getenv("ADSP_DKDV_MERGE256");
+  int v = e ? atoi(e) : 80;
+  return v < 0 ? 0 : (v > 256 ? 256 : v);
+}
+
 static int attn_common(const void* q, const void* k, const void* v, void* out, float* taus, int32_t* bmask,
                        const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D, int dtype,
                        double alpha, int is_causal, int niter, int use_hist, void* workspace, size_t workspace_bytes,
@@ -490,8 +499,10 @@ struct BwdWorkspace {
   size_t copies_bytes, queue_off, flags_off, events_off, queue2_off, kvflags_off, scratch_off, part_off, part_bytes, streams_off, dir_off, total;
   int slots;       // 0: no sparse-support kernels for these dimensions
   int dir_stride;  // offsets per stream of the hand-over table
+  int part_rows;   // rows per query head of the partial rows
+  int merge256;    // what the dK/dV kernel on the streams is launched with
 };
-static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype) {
+static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtype, int causal) {
   BwdWorkspace w = {};
   if (dtype == ADSP_F32) return w;
   w.copies_bytes = 0;
@@ -511,8 +522,16 @@ static BwdWorkspace bwd_workspace(int B, int Hq, int Hkv, int N, int D, int dtyp
     // (fp32 sums of an item worked off in parts: 32 rows of dK | dV per wave of every workgroup)
     w.scratch_off = align256(w.kvflags_off + (size_t)B * Hkv * mblocks_of(N) * 4);
     w.part_off = align256(w.scratch_off + (size_t)slots * 4 * 32 * 2 * D * 4);
-    // (with one query head per K/V head the kernel on the streams writes dK and dV itself: no partial rows)
-    w.part_bytes = (Hq == Hkv && bwd_streams_enabled()) ? 0 : (size_t)B * Hq * N * D * 4;
+    // (with one query head per K/V head the kernel on the streams writes dK and dV itself: no partial rows; with a
+    // causal mask it does so for the key blocks it merges, and the others start in front of N * merge256 / 256)
+    w.merge256 = (bwd_streams_enabled() && causal && Hq != Hkv) ? dkdv_merge256() : 0;
+    w.part_rows = N;
+    if (w.merge256 > 0) {
+      const long long bound = ((long long)N * w.merge256 + 255) / 256;
+      const long long rows = (bound + kMaskRows - 1) / kMaskRows * kMaskRows;
+      if (rows < N) w.part_rows = (int)rows;
+    }
+    w.part_bytes = (Hq == Hkv && bwd_streams_enabled()) ? 0 : (size_t)B * Hq * w.part_rows * D * 4;
     // the dQ kernel's streams, kept per (row block, wave) for the dK/dV kernel, and where their 32-key blocks start
     w.streams_off = align256(w.part_off + 2 * w.part_bytes);
     w.dir_stride = (mblocks_of(N) * 4 + 2) / 2 * 2;
@@ -544,7 +563,8 @@ typedef float reduce_f32x4 __attribute__((ext_vector_type(4)));
 template <typename T>
 __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restrict__ dk_part, const float* __restrict__ dv_part,
                                                          void* dk, void* dv, const int32_t* kv_flags, const uint32_t* ctrl2,
-                                                         const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D) {
+                                                         const void* varlen, int varlen_bits, int B, int Hq, int Hkv, int N, int D,
+                                                         int causal, int merge256, int part_rows) {
   if (ctrl2[kCtrlAllDense] != 0u) return;
   const int per_row = D / 8;
   const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -559,11 +579,12 @@ __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restric
     L = varlen_bits == 64 ? ((const long long*)varlen)[b] : (long long)((const int*)varlen)[b];
     L = L < 0 ? 0 : (L > N ? N : L);
   }
+  if (dkdv_block_merged(causal, group, row / kMaskRows * kMaskRows, (int)L, merge256)) return;  // (written by the kernel on the streams)
   float sk[8], sv[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) sk[i] = sv[i] = 0.f;
   for (int g = 0; g < (row < L ? group : 0); ++g) {
-    const size_t at = (((size_t)(b * Hq + kvh * group + g) * N) + row) * D + c * 8;
+    const size_t at = (((size_t)(b * Hq + kvh * group + g) * part_rows) + row) * D + c * 8;
     const reduce_f32x4 k0 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dk_part + at));
     const reduce_f32x4 k1 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dk_part + at + 4));
     const reduce_f32x4 v0 = __builtin_nontemporal_load(reinterpret_cast<const reduce_f32x4*>(dv_part + at));
@@ -586,7 +607,12 @@ __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restric
 
 extern "C" size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype) {
   if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
-  return adsp::bwd_workspace(B, Hq, Hkv, N, D, dtype).total;
+  return adsp::bwd_workspace(B, Hq, Hkv, N, D, dtype, 0).total;
+}
+
+extern "C" size_t adsp_attn_bwd_workspace_bytes_causal(int B, int Hq, int Hkv, int N, int D, int dtype, int is_causal) {
+  if (dtype == ADSP_F32 || B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
+  return adsp::bwd_workspace(B, Hq, Hkv, N, D, dtype, is_causal ? 1 : 0).total;
 }
 
 static int attn_bwd_impl(const void* q, const void* k, const void* v, const void* dout, const float* taus,
@@ -641,6 +667,8 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   p.dk_part = nullptr;
   p.dv_part = nullptr;
   p.part_scratch = nullptr;
+  p.merge256 = 0;
+  p.part_rows = N;
   p.streams = nullptr;
   p.stream_dir = nullptr;
   p.dir_stride = 0;
@@ -654,7 +682,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
 
   (void)hipGetLastError();
   if (dtype != ADSP_F32) {
-    w = bwd_workspace(B, Hq, Hkv, N, D, dtype);
+    w = bwd_workspace(B, Hq, Hkv, N, D, dtype, is_causal ? 1 : 0);
     const size_t need = w.total;
     if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) != 0)) return ADSP_ERR_WORKSPACE;
     // Sparse-support dQ kernel first (alpha 1.5 / 2): it serves the row blocks whose supports are short and flags the
@@ -723,6 +751,8 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
     p.hints2 = p.queue2 + 64;
     p.kv_flags = (int32_t*)(ws + w.kvflags_off);
     p.part_scratch = (float*)(ws + w.scratch_off);
+    if (p.streams) p.merge256 = w.merge256;
+    p.part_rows = w.part_rows;
     if (w.part_bytes) {
       p.dk_part = (float*)(ws + w.part_off);
       p.dv_part = (float*)(ws + w.part_off + w.part_bytes);
@@ -745,10 +775,10 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
       const dim3 grid((unsigned)((threads + 255) / 256));
       if (dtype == ADSP_BF16)
         hipLaunchKernelGGL(dkdv_reduce_kernel<bf16_t>, grid, dim3(256), 0, s, (const float*)p.dk_part, (const float*)p.dv_part, dk, dv,
-                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, varlen, varlen_bits, B, Hq, Hkv, N, D);
+                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, varlen, varlen_bits, B, Hq, Hkv, N, D, p.causal, p.merge256, p.part_rows);
       else
         hipLaunchKernelGGL(dkdv_reduce_kernel<f16_t>, grid, dim3(256), 0, s, (const float*)p.dk_part, (const float*)p.dv_part, dk, dv,
-                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, varlen, varlen_bits, B, Hq, Hkv, N, D);
+                           (const int32_t*)p.kv_flags, (const uint32_t*)p.queue2, varlen, varlen_bits, B, Hq, Hkv, N, D, p.causal, p.merge256, p.part_rows);
     }
   }
   return hipGetLastError() == hipSuccess ? ADSP_OK : ADSP_ERR_LAUNCH;

@@ -25,14 +25,16 @@ struct AttnBwdParams {
   uint32_t* hints;        // two words per K/V head: word 0 is 1 << 20 where the probe left the head to the dense kernels
   unsigned char* events;  // candidate streams, one slot per workgroup of the sparse kernel
   // the sparse-support dK/dV kernel: a control block of its own, one flag per (K/V head, key block), fp32 partial rows
-  // [B, Hq, N, D] when a K/V head serves several query heads (null otherwise), and per workgroup and wave 32 fp32
+  // [B, Hq, part_rows, D] when a K/V head serves several query heads (null otherwise), and per workgroup and wave 32 fp32
   // rows of dK | dV for the sums of an item that is worked off in parts; the streams are shared
   uint32_t* queue2;
   uint32_t* hints2;
   int32_t* kv_flags;  // [B, Hkv, n_mblk] 1 = key block left to attn_bwd_dkdv_kernel
   float* dk_part;
   float* dv_part;
+  int part_rows;  // rows per query head in dk_part / dv_part: N, or as many as the key blocks that are not merged can need
   float* part_scratch;  // [slots, waves, 32, 2 D]
+  int merge256;         // key blocks from this share (in 256ths) of a causal sequence on are served all heads in one item; 0: none
   // hand-over of the supports from the dQ kernel to the dK/dV kernel (null: the dK/dV kernel walks for itself): the dQ
   // kernel's streams kept per (row block, wave) instead of per workgroup, and per stream the offsets of the 32-key blocks
   unsigned char* streams;  // [B, Hq, n_mblk, waves, stream capacity] per member (weights, key | row << 20): the pair p / sum p, u (dP - delta) in the element type
@@ -45,5 +47,11 @@ struct AttnBwdParams {
   const float* fwd_tshift;
   const unsigned char* fwd_streams;
 };
+
+// Whether the kernel on the streams serves the key block starting at key m0 of a sequence of L keys with one item for all
+// query heads of its K/V head (then it writes dK and dV itself and the reduction over the heads leaves the block alone).
+__host__ __device__ inline bool dkdv_block_merged(int causal, int group, int m0, int L, int merge256) {
+  return merge256 > 0 && causal && group > 1 && m0 < L && (long long)m0 * 256 >= (long long)L * merge256;
+}
 
 }  // namespace adsp

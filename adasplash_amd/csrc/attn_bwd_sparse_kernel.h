@@ -1207,8 +1207,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
             *reinterpret_cast<f32x4*>(sc + D) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
             *reinterpret_cast<f32x4*>(sc + D + 4) = f32x4{acc_v[4], acc_v[5], acc_v[6], acc_v[7]};
           } else {
-            float* const o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
-            float* const o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+            const size_t part_at = ((size_t)(b * p.Hq + h) * p.part_rows + key) * D + col * 8;
+            float* const o0 = p.dk_part + part_at;
+            float* const o1 = p.dv_part + part_at;
             __builtin_nontemporal_store(f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]}, reinterpret_cast<f32x4*>(o0));
             __builtin_nontemporal_store(f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]}, reinterpret_cast<f32x4*>(o0 + 4));
             __builtin_nontemporal_store(f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]}, reinterpret_cast<f32x4*>(o1));
@@ -1325,7 +1326,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
       long long l = p.varlen_bits == 64 ? ((const long long*)p.varlen)[b] : (long long)((const int*)p.varlen)[b];
       L = (int)(l < 0 ? 0 : (l > N ? N : l));
     }
-    const bool direct = group == 1;  // a K/V head with a single query head: no sums over heads, dK and dV are written here
+    // The late key blocks of a causal sequence are short items: there one item serves all query heads of the K/V head,
+    // head after head with the sums waiting in the scratch slot, and writes dK and dV itself -- no partial rows, nothing
+    // for dkdv_reduce_kernel to add (which applies the same test).  The items of the other heads end here.
+    const bool merged = dkdv_block_merged(p.causal, group, m0, L, p.merge256);
+    if (merged && hg != 0) continue;
+    const int nh = merged ? group : 1;  // query heads of this item
+    const bool direct = group == 1 || merged;  // no sums over heads left to do: dK and dV are written here
     if (m0 >= L) {  // key block entirely inside the padding: zero gradient (dkdv_reduce_kernel writes it unless `direct`)
       if (direct) {
         constexpr int kRowDw = D * 2 / 4;
@@ -1342,14 +1349,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
     }
     // a key block that any query head gives up goes to attn_bwd_dkdv_kernel with all its heads
     int32_t* const flag = p.kv_flags + ((size_t)(b * p.Hkv + kvh) * n_mblk + mblk);
-    const size_t qo_base = ((size_t)(b * p.Hq + h) * N) * D;
     const size_t kv_base = ((size_t)(b * p.Hkv + kvh) * N) * D;
     // the row blocks whose queries can hold the block's keys in their supports
     const int rb_lo = p.causal ? mblk : 0, rb_hi = (L - 1) / BM;
     {  // no stream where the dQ kernel gave a row block up
-      const int32_t* const dq_flags = p.block_flags + (size_t)(b * p.Hq + h) * n_mblk;
       int any = s_skip;
-      for (int rb = rb_lo + tid; rb <= rb_hi; rb += SG::kThreads) any |= dq_flags[rb] != 0 ? 1 : 0;
+      for (int hh = 0; hh < nh; ++hh) {
+        const int32_t* const dq_flags = p.block_flags + (size_t)(b * p.Hq + h + hh) * n_mblk;
+        for (int rb = rb_lo + tid; rb <= rb_hi; rb += SG::kThreads) any |= dq_flags[rb] != 0 ? 1 : 0;
+      }
       if (__syncthreads_or(any)) {
         if (tid == 0) {
           *flag = 1;
@@ -1363,8 +1371,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
 #endif
     const int wave_row0 = m0 + wave * 32;
     const int k32 = wave_row0 / 32;
-    const int n_pairs = (rb_hi - rb_lo + 1) * NW;  // (row block, wave of the dQ kernel) in order
-    const size_t head_stream0 = (size_t)(b * p.Hq + h) * n_mblk * NW;  // first stream of the head
+    // (row block, wave of the dQ kernel) in order.  Where a 16-bit list entry can name a query of any head of the
+    // item (heads x N <= 65536), a merged item takes the pieces of all its heads as one sequence -- query i of head g is
+    // row g N + i from the first head's rows on -- and the sums of a part cover all heads; otherwise head follows head.
+    const int np1 = (rb_hi - rb_lo + 1) * NW;
+    const bool joint = merged && (long long)group * N <= 65536;
+    const int n_pairs = joint ? np1 * group : np1;
+    const int nh_turns = joint ? 1 : nh;
+    int part = 0;  // parts of the item so far, over all its heads
+    for (int hh = 0; hh < nh_turns; ++hh) {
+    const size_t qo_base = ((size_t)(b * p.Hq + h + hh) * N) * D;
+    const size_t head_stream0 = (size_t)(b * p.Hq + h + hh) * n_mblk * NW;  // first stream of the head
     const uint2* const src_streams = reinterpret_cast<const uint2*>(p.streams) + head_stream0 * (size_t)kSparseStreamCap;
     const uint16_t* const src_dir = p.stream_dir + head_stream0 * (size_t)p.dir_stride + k32;
 
@@ -1382,7 +1399,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
     static_assert(SG::kListCap * 4 >= 2 * kTab * 2 && SG::kListCap < 65536, "room for the table of pieces, 16-bit counts");
 
     int cursor = 0;  // next piece (wave-uniform)
-    for (int seg = 0;; ++seg) {
+    for (;; ++part) {
       // ---- the pieces of this part: as many as the lists and the table hold ----------------------------------------
       int stream_n = 0, n_tab = 0;  // wave-uniform
       const int cursor0 = cursor;   // first piece of the part
@@ -1393,8 +1410,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
           // from the last row block down: a key block holds about as many members in a row block as any other key block
           // of its head does, so the key blocks of a head that run side by side ask for the same rows of q and dO at
           // about the same time, whichever key block they are (a tenth fewer L2 misses than from the first one up)
-          const int rb = rb_hi - pi / NW, w = pi % NW;
-          const size_t sid = (size_t)rb * NW + w;
+          int hj = 0, pj = pi;  // head within the item, piece within the head
+          for (int g = 1; g < group && pj >= np1; ++g) {
+            ++hj;
+            pj -= np1;
+          }
+          const int rb = rb_hi - pj / NW, w = pj % NW;
+          const size_t sid = ((size_t)hj * n_mblk + rb) * NW + w;
           uint32_t hi = src_dir[sid * (size_t)p.dir_stride + 1];
           lo = src_dir[sid * (size_t)p.dir_stride];
           hi = hi < (uint32_t)SG::kListCap ? hi : (uint32_t)SG::kListCap;  // (what the dQ kernel wrote lies within these bounds)
@@ -1444,9 +1466,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
               if (t <= n_tab && (int)pc_incl[t - 1] <= e) a = t;
             }
             const int before = a ? (int)pc_incl[a - 1] : 0;
-            const int pi = cursor0 + a, rb = rb_hi - pi / NW, w = pi % NW;
-            ent[j] = src_streams[(uint32_t)(rb * NW + w) * (uint32_t)kSparseStreamCap + (uint32_t)pc_lo[a] + (uint32_t)(e - before)];
-            rowv[j] = (uint32_t)(rb * BM + w * 32);
+            int hj = 0, pj = cursor0 + a;
+            for (int g = 1; g < group && pj >= np1; ++g) {
+              ++hj;
+              pj -= np1;
+            }
+            const int rb = rb_hi - pj / NW, w = pj % NW;
+            ent[j] = src_streams[(uint32_t)((hj * n_mblk + rb) * NW + w) * (uint32_t)kSparseStreamCap + (uint32_t)pc_lo[a] + (uint32_t)(e - before)];
+            rowv[j] = (uint32_t)(hj * N + rb * BM + w * 32);
           }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -1578,7 +1605,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
             // the next part adds to them.  The last part writes an fp32 partial row of this query head (dkdv_reduce_kernel
             // adds up the heads of a K/V head), or dK and dV themselves where the head is the only one.
             float* const sc = p.part_scratch + (((size_t)blockIdx.x * NW + wave) * 32 + (key - wave_row0)) * (2 * D) + col * 8;
-            if (seg > 0) {
+            if (part > 0) {
               const f32x4 k0 = *reinterpret_cast<const f32x4*>(sc), k1 = *reinterpret_cast<const f32x4*>(sc + 4);
               const f32x4 v0 = *reinterpret_cast<const f32x4*>(sc + D), v1 = *reinterpret_cast<const f32x4*>(sc + D + 4);
 #pragma unroll
@@ -1589,7 +1616,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
                 acc_v[4 + i] += v1[i];
               }
             }
-            if (cursor < n_pairs) {
+            if (cursor < n_pairs || hh + 1 < nh_turns) {
               *reinterpret_cast<f32x4*>(sc) = f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]};
               *reinterpret_cast<f32x4*>(sc + 4) = f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]};
               *reinterpret_cast<f32x4*>(sc + D) = f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]};
@@ -1601,8 +1628,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
               *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dv) + kv_base + (size_t)key * D + col * 8) = wv;
             } else {
               // (streamed past the caches: the rows of q and dO that the other key blocks of the head gather stay in L2)
-              float* const o0 = p.dk_part + qo_base + (size_t)key * D + col * 8;
-              float* const o1 = p.dv_part + qo_base + (size_t)key * D + col * 8;
+              const size_t part_at = ((size_t)(b * p.Hq + h + hh) * p.part_rows + key) * D + col * 8;
+              float* const o0 = p.dk_part + part_at;
+              float* const o1 = p.dv_part + part_at;
               __builtin_nontemporal_store(f32x4{acc_k[0], acc_k[1], acc_k[2], acc_k[3]}, reinterpret_cast<f32x4*>(o0));
               __builtin_nontemporal_store(f32x4{acc_k[4], acc_k[5], acc_k[6], acc_k[7]}, reinterpret_cast<f32x4*>(o0 + 4));
               __builtin_nontemporal_store(f32x4{acc_v[0], acc_v[1], acc_v[2], acc_v[3]}, reinterpret_cast<f32x4*>(o1));
@@ -1647,13 +1675,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_W
           }
         }
       }
-      if (cursor >= n_pairs) break;
+      if (cursor >= n_pairs && hh + 1 == nh_turns) break;
       // (the sums just written to the scratch slot are read back by the next part, by this wave: its stores have landed
       // before the next part begins; every lane is done with the lists)
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       __builtin_amdgcn_wave_barrier();
+      if (cursor >= n_pairs) {
+        ++part;
+        break;
+      }
     }
+    }  // (heads of the item)
   }
 }
 

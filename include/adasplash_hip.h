@@ -189,8 +189,17 @@ int adsp_attn_bwd_kept(const void* q, const void* k, const void* v, const void* 
  * none where Hq == Hkv), and the supports the dq kernel hands to the dk/dv kernel: per query row block of 128 rows
  * 51 KiB of (weights, key) pairs and a table of 4 * ceil(N / 128) + 2 16-bit offsets per wave.
  * 16-byte aligned device memory; contents need not survive between calls; concurrent calls need a buffer each.
+ * This is the size that serves any call with these dimensions.
  */
 size_t adsp_attn_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D, int dtype);
+
+/*
+ * The same for a call whose is_causal is known: with a causal mask the dk/dv kernel serves the later key blocks of a
+ * sequence (from 5/16 of its length on) for all query heads of a K/V head at once and needs partial rows for the first
+ * ones only (about 5/16 of the bytes above), so the workspace is smaller.  adsp_attn_bwd and adsp_attn_bwd_kept accept a
+ * workspace of either size.  (No counterpart in the reference, which allocates inside its backward.)
+ */
+size_t adsp_attn_bwd_workspace_bytes_causal(int B, int Hq, int Hkv, int N, int D, int dtype, int is_causal);
 
 /*
  * Backward of both attention variants: dq, dk, dv for the upstream gradient dout.

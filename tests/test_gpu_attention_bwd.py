@@ -210,6 +210,54 @@ def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B
         assert max_err(a, b.float().cpu(), report=False) < grad_tol(dtype)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,N,D,dtype,lens,with_oracle", [
+    (2, 8, 2, 1024, 64, torch.bfloat16, [1024, 700], True),   # 4 heads x 1024 rows: one 16-bit list entry names any of them
+    (1, 4, 1, 3000, 128, torch.float16, [2777], True),
+    (1, 16, 1, 4224, 64, torch.bfloat16, [4100], False),      # 16 x 4224 > 65536: head after head, sums in the scratch slot
+])
+def test_late_key_blocks_served_for_all_query_heads_at_once(B, Hq, Hkv, N, D, dtype, lens, with_oracle):
+    """With a causal mask the dK/dV kernel on the streams serves the key blocks from 5/16 of a sequence on with one item
+    for all query heads of a K/V head and writes dK and dV itself (ADSP_DKDV_MERGE256, default 80); the earlier blocks
+    go per query head through fp32 partial rows and the reduction.  0 turns the merging off, 1 merges every block but
+    the first (long items that are worked off in parts).  All three must agree -- the same members and weights, summed
+    in another order -- and meet the oracle where it is affordable."""
+    import os
+    varlen = torch.tensor(lens, dtype=torch.int32)
+    old = os.environ.get("ADSP_DKDV_MERGE256")
+    got = {}
+    want = None
+    try:
+        for mode in ("80", "0", "1"):
+            os.environ["ADSP_DKDV_MERGE256"] = mode
+            if with_oracle:
+                got[mode], want = run_case(1.5, True, B, Hq, Hkv, N, D, dtype, varlen=varlen, version=2, seed=11)
+                check(got[mode], want, dtype)
+            else:
+                g = torch.Generator().manual_seed(11)
+                q = torch.randn(B, Hq, N, D, generator=g).to(dtype)
+                k = torch.randn(B, Hkv, N, D, generator=g).to(dtype)
+                v = torch.randn(B, Hkv, N, D, generator=g).to(dtype)
+                do = torch.randn(B, Hq, N, D, generator=g).to(dtype)
+                qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+                A.adasplash_v2(qg, kg, vg, niter=10, varlen=varlen.to(DEV)).backward(do.to(DEV))
+                got[mode] = (qg.grad, kg.grad, vg.grad)
+                assert all(torch.isfinite(t).all() for t in got[mode])
+    finally:
+        if old is None:
+            os.environ.pop("ADSP_DKDV_MERGE256", None)
+        else:
+            os.environ["ADSP_DKDV_MERGE256"] = old
+    for mode in ("0", "1"):
+        for a, b in zip(got["80"], got[mode]):
+            # (fp32 sums of the same terms in another order, rounded once to the element type)
+            assert max_err(a, b.float().cpu(), report=False) < 0.25 * grad_tol(dtype), mode
+    from adasplash_amd import _lib
+    lib = _lib.load()
+    dt = _lib.dtype_code(got["80"][0])
+    assert lib.adsp_attn_bwd_workspace_bytes_causal(B, Hq, Hkv, N, D, dt, 1) < lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dt)
+    assert lib.adsp_attn_bwd_workspace_bytes_causal(B, Hq, Hkv, N, D, dt, 0) == lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, dt)
+
+
 @pytest.mark.parametrize("alpha,causal,B,Hq,Hkv,N,D,dtype,lens,version,scale,sparse", [
     (1.5, True, 2, 4, 2, 1024, 128, torch.bfloat16, [1024, 700], 2, 1.0, "1"),
     (1.5, True, 1, 2, 1, 3000, 64, torch.float16, [2777], 2, 1.0, "1"),

@@ -181,6 +181,11 @@ def test_sizing_helpers_and_status_strings():
     assert lib.adsp_attn_supports_bytes(8, 32, 8, 8192, 128, _lib.ADSP_F32) == 0
     assert lib.adsp_attn_supports_bytes(2, 2, 2, 100, 32, _lib.ADSP_F16) == 0
     assert lib.adsp_attn_bwd_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16) > 2 * 8 * 32 * 8192 * 128 * 4 + items * slot
+    # with a causal mask the later key blocks need no partial rows: 5/16 of them are left
+    any_mask = lib.adsp_attn_bwd_workspace_bytes(8, 32, 8, 8192, 128, _lib.ADSP_BF16)
+    assert lib.adsp_attn_bwd_workspace_bytes_causal(8, 32, 8, 8192, 128, _lib.ADSP_BF16, 0) == any_mask
+    assert lib.adsp_attn_bwd_workspace_bytes_causal(8, 32, 8, 8192, 128, _lib.ADSP_BF16, 1) == any_mask - 2 * 8 * 32 * (8192 - 2560) * 128 * 4
+    assert lib.adsp_attn_bwd_workspace_bytes_causal(8, 8, 8, 8192, 128, _lib.ADSP_BF16, 1) == lib.adsp_attn_bwd_workspace_bytes(8, 8, 8, 8192, 128, _lib.ADSP_BF16)
     assert lib.adsp_status_string(0) == b"ok"
     assert all(len(lib.adsp_status_string(s)) > 0 for s in range(0, 9))
 
