@@ -210,12 +210,13 @@ def test_dkdv_from_the_dq_kernels_streams_and_from_its_own_walk(alpha, causal, B
         assert max_err(a, b.float().cpu(), report=False) < grad_tol(dtype)
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,N,D,dtype,lens,with_oracle", [
-    (2, 8, 2, 1024, 64, torch.bfloat16, [1024, 700], True),   # 4 heads x 1024 rows: one 16-bit list entry names any of them
-    (1, 4, 1, 3000, 128, torch.float16, [2777], True),
-    (1, 16, 1, 4224, 64, torch.bfloat16, [4100], False),      # 16 x 4224 > 65536: head after head, sums in the scratch slot
+@pytest.mark.parametrize("B,Hq,Hkv,N,D,dtype,lens,with_oracle,scale", [
+    (2, 8, 2, 1024, 64, torch.bfloat16, [1024, 700], True, 1.0),   # 4 heads x 1024 rows: one 16-bit list entry names any of them
+    (1, 4, 1, 3000, 128, torch.float16, [2777], True, 1.0),
+    (1, 4, 2, 2048, 128, torch.bfloat16, [2048], True, 0.55),      # long supports: some row blocks, and their key blocks, go to the dense kernels
+    (1, 16, 1, 4224, 64, torch.bfloat16, [4100], False, 1.0),      # 16 x 4224 > 65536: head after head, sums in the scratch slot
 ])
-def test_late_key_blocks_served_for_all_query_heads_at_once(B, Hq, Hkv, N, D, dtype, lens, with_oracle):
+def test_late_key_blocks_served_for_all_query_heads_at_once(B, Hq, Hkv, N, D, dtype, lens, with_oracle, scale):
     """With a causal mask the dK/dV kernel on the streams serves the key blocks from 5/16 of a sequence on with one item
     for all query heads of a K/V head and writes dK and dV itself (ADSP_DKDV_MERGE256, default 80); the earlier blocks
     go per query head through fp32 partial rows and the reduction.  0 turns the merging off, 1 merges every block but
@@ -230,7 +231,7 @@ def test_late_key_blocks_served_for_all_query_heads_at_once(B, Hq, Hkv, N, D, dt
         for mode in ("80", "0", "1"):
             os.environ["ADSP_DKDV_MERGE256"] = mode
             if with_oracle:
-                got[mode], want = run_case(1.5, True, B, Hq, Hkv, N, D, dtype, varlen=varlen, version=2, seed=11)
+                got[mode], want = run_case(1.5, True, B, Hq, Hkv, N, D, dtype, varlen=varlen, version=2, seed=11, scale=scale)
                 check(got[mode], want, dtype)
             else:
                 g = torch.Generator().manual_seed(11)
