@@ -556,7 +556,8 @@ __global__ __launch_bounds__(256) void bwd_ctrl_clear_kernel(uint32_t* ctrl2, co
 }
 
 // dK, dV = sum over the query heads of a K/V head of the sparse-support kernel's fp32 partial rows; key blocks left to
-// attn_bwd_dkdv_kernel are skipped (that kernel writes them).  A thread adds up 8 columns of
+// attn_bwd_dkdv_kernel are skipped (that kernel writes them), and so are those the kernel on the streams served for all
+// heads at once.  A thread adds up 8 columns of
 // one key row.  Rows past the valid length are zeros and their partial rows are not read (the key blocks that lie
 // wholly in the padding have none).
 typedef float reduce_f32x4 __attribute__((ext_vector_type(4)));

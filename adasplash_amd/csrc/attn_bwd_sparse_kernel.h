@@ -1252,8 +1252,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_SPARSE
 // its lists hold works them off in parts (the sums wait in fp32 in the workgroup's scratch slot); the waves of a
 // workgroup share nothing and do not wait for each other.  The sums are fp32 partial rows per query head for
 // dkdv_reduce_kernel; where a K/V head has a single query head the last part writes dK and dV in the element type and
-// there is no reduction.  A key block one of whose row blocks the dQ kernel gave up (no stream) is flagged for
-// attn_bwd_dkdv_kernel with all its heads.
+// there is no reduction.  With a causal mask the later key blocks of a sequence (dkdv_block_merged) are short: there
+// one item serves all query heads of the K/V head and writes dK and dV itself.  A key block one of whose row blocks the
+// dQ kernel gave up (no stream) is flagged for attn_bwd_dkdv_kernel with all its heads.
 template <typename T, int D, int AM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ADSP_DKDV_WAVES, ADSP_DKDV_WAVES))) void attn_bwd_dkdv_stream_kernel(AttnBwdParams p) {
   constexpr int kQuads = ADSP_DKDV_QUADS;

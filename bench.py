@@ -35,10 +35,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these
 # same workloads, each counter scaled by what it reads for a plain 1 GiB copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the summaries are in profiles/.  None = not measured.
-MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.472e9, "c3": 0.5074e9, "c5": 0.556e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5370e9,
+MEASURED_HBM_TRAFFIC_BYTES = {"c4": 2.467e9, "c3": 0.5076e9, "c5": 0.556e9, "c2_f32": 1.0739e9, "c2_bf16": 0.5370e9,
                               "c2_bwd_f32": 1.0847e9, "c2_bwd_bf16": 0.5476e9,
-                              "c4_bwd": 10.92e9,
-                              "c5_bwd": 0.836e9}  # c4_bwd: sparse dq kernel 3.21e9 + dk/dv kernel on its streams 5.97e9 + reduction 1.74e9
+                              "c4_bwd": 12.57e9,
+                              "c5_bwd": 0.795e9}  # c4_bwd: sparse dq kernel 3.21e9 + dk/dv kernel on its streams 8.75e9 + reduction 0.61e9
 
 
 # The kernel that dominates a forward step of each workload.  A 16-bit step of the v2 entry point is four launches: a

@@ -18,6 +18,9 @@
  *                                   the dQ kernel's candidate streams
  *       ADSP_PROBE_MAX_SUPPORT=n    the support the probe lets a K/V head's longest rows have before it
  *                                   leaves the head to the dense kernels (default 28; 0: every head)
+ *       ADSP_DKDV_MERGE256=n        the share of a causal sequence, in 256ths, from which on the dK/dV kernel serves
+ *                                   a key block for all query heads of a K/V head at once (default 80; 0: never).
+ *                                   Sizes the backward workspace too: the same value for the size query and the call.
  *
  * The entry points replace the Triton launches inside the reference's autograd wrappers (the
  * reference has no FFI of its own; these are the calls a binding would make in their place):
