@@ -190,6 +190,25 @@ def test_sizing_helpers_and_status_strings():
     assert all(len(lib.adsp_status_string(s)) > 0 for s in range(0, 9))
 
 
+def test_backward_workspace_for_a_causal_call_follows_the_merge_border(monkeypatch):
+    """With a causal mask and several query heads per K/V head the partial rows cover the key blocks in front of
+    N * ADSP_DKDV_MERGE256 / 256 only (rounded up to whole 128-key blocks); the rest of the workspace is the same."""
+    lib = _lib.load()
+    B, Hq, Hkv, D = 2, 8, 2, 64
+    for N in (128, 1000, 4096, 8192, 65536):
+        for m256 in (0, 1, 64, 80, 200, 256):
+            monkeypatch.setenv("ADSP_DKDV_MERGE256", str(m256))
+            full = lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hkv, N, D, _lib.ADSP_BF16)
+            causal = lib.adsp_attn_bwd_workspace_bytes_causal(B, Hq, Hkv, N, D, _lib.ADSP_BF16, 1)
+            rows = N
+            if m256 > 0:
+                bound = (N * m256 + 255) // 256
+                rows = min(N, (bound + 127) // 128 * 128)
+            assert full - causal == 2 * B * Hq * (N - rows) * D * 4, (N, m256)
+            assert lib.adsp_attn_bwd_workspace_bytes_causal(B, Hq, Hkv, N, D, _lib.ADSP_BF16, 0) == full
+            assert lib.adsp_attn_bwd_workspace_bytes_causal(B, Hq, Hq, N, D, _lib.ADSP_BF16, 1) == lib.adsp_attn_bwd_workspace_bytes(B, Hq, Hq, N, D, _lib.ADSP_BF16)
+
+
 def test_argument_errors_come_back_as_status_codes():
     lib = _lib.load()
     # no pointer is dereferenced and nothing is launched for these
